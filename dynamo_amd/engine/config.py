@@ -16,7 +16,7 @@ from typing import Optional
 @dataclass
 class ModelConfig:
     name: str = "llama-3-8b"
-    arch: str = "llama"            # llama | opt | mixtral | qwen2 | bolatar | fironex
+    arch: str = "llama"            # llama | opt | mixtral | qwen2 | bolatar | fironex | kefesun
     hidden_size: int = 4096
     intermediate_size: int = 14336
     num_layers: int = 32
@@ -39,12 +39,13 @@ class ModelConfig:
     learned_pos_emb: bool = False
     # qwen2-style QKV bias
     attn_bias: bool = False
-    # layer-list models (bolatar, fironex): one dict per layer with its mixer type,
+    # layer-list models (bolatar, fironex, kefesun): one dict per layer with its mixer type,
     # mixer sizes and feed-forward, as in the checkpoint's config.json
     layer_specs: Optional[list] = None
     embed_scale: float = 1.0       # multiplies token embeddings
     logit_softcap: float = 0.0     # cap * tanh(logits / cap); 0 = off
     residual_mult: float = 1.0     # scales a normed sublayer output (fironex)
+    conv_taps: int = 0             # taps of the sublayers' input convolution (kefesun)
     # local HF checkpoint dir to load real weights from ("" = random init)
     weights_path: str = ""
 
@@ -162,6 +163,33 @@ PRESETS = {
                         "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0,
                                     "original": 64}}},
              "mlp": {"kind": "dense", "ff": 100}},
+        ]),
+    # layer-list model with an input convolution on every sublayer: sigmoid
+    # attention under a window that keeps the first tokens, a minimal gated
+    # recurrent unit, routed experts with identity and shared experts
+    "tiny-kefesun": ModelConfig(
+        name="tiny-kefesun", arch="kefesun", hidden_size=80, vocab_size=150,
+        num_layers=3, rms_eps=1e-5, embed_scale=3.0, conv_taps=3,
+        tie_embeddings=True, norm="layernorm", intermediate_size=0,
+        num_q_heads=1, num_kv_heads=1, head_dim=1,
+        layer_specs=[
+            {"type": "attention", "mixer": {
+                "heads": 6, "kv_heads": 2, "dim": 24, "vdim": 16,
+                "scale": 0.2, "mask": {"size": 20, "keep_first": 3},
+                "rot": {"base": 10000.0, "dims": 12}},
+             "mlp": {"kind": "moe", "expert": {"ff": 40},
+                     "router": {"experts": 5, "identity": 1, "top": 3,
+                                "scale": 1.5,
+                                "groups": {"count": 3, "keep": 2}},
+                     "shared": {"ff": 56}}},
+            {"type": "mingru", "mixer": {"width": 72}, "mlp": None},
+            {"type": "attention", "mixer": {
+                "heads": 2, "kv_heads": 1, "dim": 16, "vdim": 24,
+                "scale": 0.25, "rot": {"base": 500.0, "dims": 16}},
+             "mlp": {"kind": "moe", "expert": {"ff": 48},
+                     "router": {"experts": 4, "identity": 0, "top": 2,
+                                "scale": 1.0},
+                     "shared": None}},
         ]),
 }
 

@@ -2,7 +2,9 @@
 slot-addressed fp32 state (matrix memories, a gated linear unit), and
 softmax attention over the paged cache with a distance bias / query
 temperature / value norm, with differential heads under a sliding window,
-or over a shared compressed latent.
+or over a shared compressed latent; attention with unnormalised sigmoid
+weights under a window that keeps the first tokens; a minimal gated
+recurrent unit; and a routed mixture of small feed-forward experts.
 
 Every mixer takes the normed hidden rows h [T, W] of the engine's flat
 batch and a `MixContext` (sequence spans, state tensors of its layer, cache
@@ -565,3 +567,189 @@ class XIELUMLP(torch.nn.Module):
     def forward(self, h):
         return F.linear(sops.xielu(F.linear(h, self.w_up), self.act),
                         self.w_down)
+
+
+class SigmoidAttention(torch.nn.Module):
+    """Grouped-query attention whose weight of a visible key is
+    sigmoid(scale q.k + b_h), not normalised over the keys. q, k, v carry
+    biases; q and k are RMS-normed per head (one weight of the head size for
+    all heads), then rotated over their first rot.dims entries (pairs
+    (i, i + dims/2), or interleaved). Row i sees key j <= i when
+    i - j < window or j < keep_first; window None = every earlier key."""
+
+    def __init__(self, width, heads, kv_heads, dim, vdim, scale, rot, window,
+                 keep_first, eps, init, interleaved=False, sigmoid=True):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("query heads must be a multiple of kv heads")
+        self.W, self.H, self.G, self.dk, self.dv = width, heads, kv_heads, dim, vdim
+        self.scale, self.eps = scale, eps
+        self.window, self.keep_first = int(window or 0), int(keep_first or 0)
+        self.interleaved, self.sigmoid = interleaved, sigmoid
+        self.off_k = heads * dim
+        self.off_v = self.off_k + kv_heads * dim
+        # fused rows: q | k | v, each with its bias
+        self.w_in = init.mat(self.off_v + kv_heads * vdim, width)
+        self.b_in = init.vec(self.off_v + kv_heads * vdim, -0.2, 0.2).to(
+            init.dtype)
+        self.q_norm = init.vec(dim, 0.7, 1.3)
+        self.k_norm = init.vec(dim, 0.7, 1.3)
+        self.freqs = None
+        if rot:
+            self.freqs = rotary_frequencies(rot).to(init.device)
+            if 2 * self.freqs.shape[1] > dim:
+                raise ValueError("rotary dims exceed the head size")
+        self.head_bias = init.vec(heads, -3.0, -1.0)
+        self.w_o = init.mat(width, heads * vdim)
+
+    def state_shapes(self):
+        return []
+
+    def kv_shape(self):
+        return (self.G, self.dk, self.dv)
+
+    def load(self, get: Getter):
+        _put(self.w_in, torch.cat([get("q"), get("k"), get("v")], 0))
+        _put(self.b_in, torch.cat([get("q.b"), get("k.b"), get("v.b")], 0))
+        _put(self.q_norm, get("q.norm"))
+        _put(self.k_norm, get("k.norm"))
+        _put(self.head_bias, get("pb"))
+        _put(self.w_o, get("o"))
+
+    def forward(self, h, ctx: MixContext):
+        proj = F.linear(h, self.w_in, self.b_in)
+        sops.headnorm_rope_append(
+            proj, self.H, self.G, self.dk, self.dv, self.off_k, self.off_v,
+            self.q_norm, self.k_norm, self.freqs, self.interleaved, self.eps,
+            ctx.positions, ctx.kcache, ctx.vcache, ctx.slot_mapping)
+        y = sops.paged_attention_rows(
+            proj, 0, self.H, 1, ctx.kcache, ctx.vcache, self.dv,
+            ctx.positions, ctx.sb, self.scale, self.window, self.keep_first,
+            self.head_bias, self.sigmoid, out_dtype=h.dtype)
+        return F.linear(y.view(h.shape[0], self.H * self.dv), self.w_o)
+
+
+class MinGRUMixer(torch.nn.Module):
+    """Minimal gated recurrent unit: gate z = sigmoid(W_z h + b_z) and
+    candidate c(W_x h + b_x) read the current token only (c(u) = u + 1/2 for
+    u >= 0, sigmoid(u) below); S <- (1 - z) S + z c per channel in fp32;
+    output W_o (S * silu(W_g h))."""
+
+    def __init__(self, width, channels, init):
+        super().__init__()
+        self.W, self.C = width, channels
+        # fused rows: z | x | g (the output gate has no bias)
+        self.w_in = init.mat(3 * channels, width)
+        self.b_in = torch.cat([init.vec(2 * channels, -0.5, 0.5),
+                               torch.zeros(channels, device=init.device)]
+                              ).to(init.dtype)
+        self.w_o = init.mat(width, channels)
+
+    def state_shapes(self):
+        return [(self.C,)]
+
+    def kv_shape(self):
+        return None
+
+    def load(self, get: Getter):
+        _put(self.w_in, torch.cat([get("z"), get("x"), get("g")], 0))
+        b = torch.cat([get("z.b"), get("x.b")], 0)
+        _put(self.b_in, torch.cat([b, torch.zeros(self.C, dtype=b.dtype)], 0))
+        _put(self.w_o, get("o"))
+
+    def forward(self, h, ctx: MixContext):
+        proj = F.linear(h, self.w_in, self.b_in)
+        y = sops.mingru_scan(proj, self.C, ctx.states[0], ctx.sb, h.dtype)
+        return F.linear(y, self.w_o)
+
+
+class RoutedExperts(torch.nn.Module):
+    """Mixture of feed-forward experts W_down relu(W_up h)^2 without biases.
+    The router (fp32) scores all its outputs with a softmax; the `top`
+    outputs with the largest corrected scores are chosen, among the `keep`
+    best of `groups` equal groups of neighbouring outputs; the chosen ones
+    weigh in with their uncorrected score times `scale`. The last `identity`
+    router outputs are identity experts (output = input). A shared expert of
+    the same form, when present, runs for every token.
+
+    Chosen (token, expert) pairs get a row of a gathered batch - expert e
+    owns rows base[e] + rank - so that each expert is one GEMM over its
+    rows: per expert when the counts are read on the host (prompts), or one
+    batched GEMM over fixed-capacity blocks without any host read (few
+    rows: decoding, graph capture)."""
+
+    PADDED_MAX_ROWS = 64
+
+    def __init__(self, width, experts, ff, top, scale, identity, groups, keep,
+                 shared_ff, init):
+        super().__init__()
+        n = experts + identity
+        if n % groups or not 1 <= keep <= groups:
+            raise ValueError("router outputs must divide into their groups")
+        if top > keep * (n // groups):
+            raise ValueError("more experts per token than the kept groups hold")
+        self.W, self.E, self.n, self.ff = width, experts, n, ff
+        self.top, self.scale = top, scale
+        self.groups, self.keep = groups, keep
+        f32 = dict(dtype=torch.float32, device=init.device)
+        self.router = (torch.randn(n, width, generator=init.gen)
+                       * width ** -0.5).to(**f32)
+        self.correction = init.vec(n, -0.05, 0.05)
+        self.w_up = torch.stack([init.mat(ff, width) for _ in range(experts)])
+        self.w_down = torch.stack([init.mat(width, ff) for _ in range(experts)])
+        self.shared_up = self.shared_down = None
+        if shared_ff:
+            self.shared_up = init.mat(shared_ff, width)
+            self.shared_down = init.mat(width, shared_ff)
+        self._pad_base = {}
+
+    def load(self, get: Getter):
+        _put(self.router, get("router"))
+        _put(self.correction, get("correction"))
+        _put(self.w_up, torch.stack([get(f"e{e}.up") for e in range(self.E)]))
+        _put(self.w_down,
+             torch.stack([get(f"e{e}.down") for e in range(self.E)]))
+        if self.shared_up is not None:
+            _put(self.shared_up, get("shared.up"))
+            _put(self.shared_down, get("shared.down"))
+
+    def _padded_base(self, cap, device):
+        key = (cap, str(device))
+        if key not in self._pad_base:
+            self._pad_base[key] = (torch.arange(self.n, dtype=torch.int32)
+                                   * cap).to(device)
+        return self._pad_base[key]
+
+    def forward(self, h):
+        T, E = h.shape[0], self.E
+        logits = F.linear(h.float(), self.router)
+        idx, wgt = sops.moe_route(logits, self.correction, self.groups,
+                                  self.keep, self.top, self.scale)
+        rank, counts = sops.moe_dispatch(idx, self.n)
+        if T <= self.PADDED_MAX_ROWS:
+            # every expert gets a block of T rows: static shapes, no host read
+            base = self._padded_base(T, h.device)
+            xg = sops.moe_gather(h, idx, rank, base, E, E * T)
+            a = sops.relu_squared(torch.bmm(xg.view(E, T, self.W),
+                                            self.w_up.transpose(1, 2)))
+            y = torch.bmm(a, self.w_down.transpose(1, 2)).view(E * T, self.W)
+        else:
+            cnt = counts[:E].tolist()
+            base = torch.zeros(E + 1, dtype=torch.int32, device=h.device)
+            base[1:] = torch.cumsum(counts[:E], 0).to(torch.int32)
+            rows = sum(cnt)
+            xg = sops.moe_gather(h, idx, rank, base, E, rows)
+            y = torch.empty(rows, self.W, dtype=h.dtype, device=h.device)
+            r0 = 0
+            for e, n in enumerate(cnt):
+                if n:
+                    a = sops.relu_squared(F.linear(xg[r0:r0 + n],
+                                                   self.w_up[e]))
+                    y[r0:r0 + n] = F.linear(a, self.w_down[e])
+                r0 += n
+        shared = None
+        if self.shared_up is not None:
+            shared = F.linear(sops.relu_squared(F.linear(h, self.shared_up)),
+                              self.shared_down)
+        return sops.moe_combine(y, h, idx, wgt, rank, base, E, shared,
+                                h.dtype)

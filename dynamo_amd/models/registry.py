@@ -20,13 +20,17 @@ def build_model(cfg: ModelConfig, device, dtype, tp=None, seed: int = 0):
     if cfg.arch == "fironex":
         from .fironex import FironexForCausalLM
         return FironexForCausalLM(cfg, device, dtype, tp, seed)
+    if cfg.arch == "kefesun":
+        from .kefesun import KefesunForCausalLM
+        return KefesunForCausalLM(cfg, device, dtype, tp, seed)
     raise ValueError(f"unknown arch {cfg.arch}")
 
 
 # config.json "architecture" values of layer-list checkpoints -> the module
 # whose config_from_json reads them
 LAYER_LIST_ARCHS = {"bolatar": "dynamo_amd.models.bolatar",
-                    "fironex": "dynamo_amd.models.fironex"}
+                    "fironex": "dynamo_amd.models.fironex",
+                    "kefesun": "dynamo_amd.models.kefesun"}
 
 
 def native_extensions(cfg: ModelConfig, device: str):

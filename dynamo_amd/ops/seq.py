@@ -291,37 +291,44 @@ def latent_append(cache, z, z_col: int, norm_w, slot_mapping, positions,
 
 def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
                          dv: int, positions, sb: SeqBatch, scale: float,
-                         window: int = 0):
-    """Causal softmax attention of every row over its sequence's pages.
-    -> fp32 [T, H, kmaps, dv]. Queries lie in q at off_q as [H][kmaps][dk];
-    kcache [P, G, ps, kmaps * dk]; values from vcache [P, G, ps, dv] or,
-    without one, from the first dv entries of the key rows. window > 0:
-    row i sees keys j with 0 <= i - j < window."""
+                         window: int = 0, keep_first: int = 0, head_bias=None,
+                         sigmoid: bool = False, out_dtype=torch.float32):
+    """Causal attention of every row over its sequence's pages.
+    -> [T, H, kmaps, dv] (fp32 unless out_dtype says otherwise). Queries lie
+    in q at off_q as [H][kmaps][dk]; kcache [P, G, ps, kmaps * dk]; values
+    from vcache [P, G, ps, dv] or, without one, from the first dv entries of
+    the key rows. window > 0: row i sees keys j with 0 <= i - j < window,
+    and also the keys j < keep_first whatever their distance. head_bias
+    (fp32 [H]) is added to the scaled scores. The weights are a softmax over
+    the visible keys, or with `sigmoid` the plain sigmoid of each score
+    (not normalised over the keys)."""
     if q.is_cuda:
         T = q.shape[0]
-        out = torch.empty(T, H, kmaps, dv, dtype=torch.float32,
-                          device=q.device)
+        out = torch.empty(T, H, kmaps, dv, dtype=out_dtype, device=q.device)
         m = hip_seq()
         # bf16 rows whose sizes fit go to the matrix cores: prompt portions
         # as 64-row tiles, decoded tokens (rows [0, num_decode)) with their
         # heads as tile rows when at least 8 heads share a kv head. fp32,
         # other sizes and the remaining rows take the row kernel.
         krow, G = kcache.shape[3], kcache.shape[1]
+        f32out = out_dtype == torch.float32
         fits = (q.dtype == torch.bfloat16
-                and m.paged_attention_mfma_supported(krow // kmaps, dv, True)
+                and m.paged_attention_mfma_supported(krow // kmaps, dv, f32out)
                 and krow % 8 == 0 and kcache.data_ptr() % 16 == 0
                 and (vcache is None or vcache.data_ptr() % 16 == 0))
         tiled = fits and sb.tiles is not None
         ndec = min(sb.num_decode, T)
         done = 0
-        if fits and ndec and H // G >= 8:
+        opts = (int(window), int(keep_first), head_bias, bool(sigmoid))
+        if (fits and ndec and H // G >= 8 and f32out
+                and m.paged_attention_mfma_supported(krow // kmaps, dv, True)):
             nsplit = max(1, min(16, 512 // (ndec * G * kmaps)))
             part = torch.empty(ndec, H, kmaps, nsplit, dv + 2,
                                dtype=torch.float32, device=q.device)
             m.paged_attention_mfma_decode(
                 out[:ndec], part, q[:ndec], off_q, kcache, vcache,
                 sb.page_table, sb.tok_seq[:ndec], positions[:ndec],
-                sb.seq_len, float(scale), int(kmaps), int(window))
+                sb.seq_len, float(scale), int(kmaps), *opts)
             done = ndec
         end = ndec if tiled else T
         if end > done:
@@ -329,15 +336,16 @@ def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
                 out[done:end], q[done:end], off_q, kcache, vcache,
                 sb.page_table, sb.tok_seq[done:end], positions[done:end],
                 sb.seq_len, None, None, float(scale), 0.0, 1, int(kmaps),
-                int(window))
+                *opts)
         if tiled and sb.tiles[0].numel():
             m.paged_attention_mfma(
                 out, q, off_q, kcache, vcache, sb.page_table, sb.tiles[0],
                 sb.tiles[1], 64, sb.tok_seq, positions, None, None,
-                float(scale), 0.0, 1, int(kmaps), int(window))
+                float(scale), 0.0, 1, int(kmaps), *opts)
         return out
-    return seq_ref.paged_attention_rows(q, off_q, H, kmaps, kcache, vcache,
-                                        dv, positions, sb, scale, window)
+    return seq_ref.paged_attention_rows(
+        q, off_q, H, kmaps, kcache, vcache, dv, positions, sb, scale, window,
+        keep_first, head_bias, sigmoid).to(out_dtype)
 
 
 def diff_norm_gate(a, lam, post: float, gate, eps: float, out_dtype):
@@ -388,3 +396,118 @@ def rglru_scan(u, gates, br, bi, lam, y, state, sb: SeqBatch, decay: float,
         return out
     return seq_ref.rglru_scan(u, gates, br, bi, lam, y, state, sb, decay,
                               out_dtype)
+
+
+# -- input convolution of a sublayer, normed rotated heads into the cache,
+# -- minimal gated recurrence, routed experts ---------------------------------
+def residual_conv(res, w, conv_state, sb: SeqBatch, out_dtype):
+    """res + conv(res): a short causal per-channel convolution over the fp32
+    rows res [T, W] (w fp32 [W, taps], the last tap weighs the current
+    token, no bias), added to its own input. The slot's saved rows
+    [slots, taps - 1, W] continue earlier portions and are updated."""
+    if res.is_cuda:
+        out = torch.empty(res.shape, dtype=out_dtype, device=res.device)
+        hip_seq().residual_conv(out, res, w, conv_state, sb.tok_seq,
+                                *_args(sb))
+        return out
+    return seq_ref.residual_conv(res, w, conv_state, sb, out_dtype)
+
+
+def headnorm_rope_append(proj, H: int, G: int, dk: int, dv: int, off_k: int,
+                         off_v: int, qw, kw, freqs, interleaved: bool,
+                         eps: float, positions, kcache, vcache, slot_mapping):
+    """Per token row of proj (q at column 0 as [H][dk], k at off_k as
+    [G][dk], v at off_v as [G][dv]): every query and key vector is divided
+    by its root mean square, multiplied by qw / kw (fp32 [dk], shared by the
+    heads) and has its first rot dims rotated by position * f (freqs as in
+    rope_rows; None = no rotation). Queries are rewritten in place; keys and
+    the raw values go to the token's cache slot."""
+    if proj.is_cuda:
+        hip_seq().headnorm_rope_append(
+            proj, H, G, dk, dv, off_k, off_v, qw, kw, freqs,
+            bool(interleaved), float(eps), positions, kcache, vcache,
+            slot_mapping)
+    else:
+        seq_ref.headnorm_rope_append(
+            proj, H, G, dk, dv, off_k, off_v, qw, kw, freqs, interleaved,
+            eps, positions, kcache, vcache, slot_mapping)
+
+
+def _longest(sb: SeqBatch, T: int) -> int:
+    """Upper bound of the longest portion of the step (known on the host,
+    or all rows)."""
+    if sb.host is not None:
+        return max(1, max((n for _s, n, _l, _p in sb.host), default=1))
+    return max(1, T)
+
+
+def mingru_scan(proj, C: int, state, sb: SeqBatch, out_dtype):
+    """Minimal gated recurrent unit over proj [T, 3C] = z | u | g
+    pre-activations: S <- (1 - sigmoid(z)) S + sigmoid(z) c(u) with
+    c(u) = u + 1/2 for u >= 0 and sigmoid(u) below; returns S * silu(g).
+    state fp32 [slots, C]."""
+    if proj.is_cuda:
+        out = torch.empty(proj.shape[0], C, dtype=out_dtype,
+                          device=proj.device)
+        hip_seq().mingru_scan(out, proj, state, *_args(sb),
+                              _longest(sb, proj.shape[0]))
+        return out
+    return seq_ref.mingru_scan(proj, C, state, sb, out_dtype)
+
+
+def relu_squared(x):
+    if x.is_cuda:
+        out = torch.empty_like(x)
+        hip_seq().relu_squared(out, x)
+        return out
+    return seq_ref.relu_squared(x)
+
+
+def moe_route(logits, correction, groups: int, keep: int, top: int,
+              scale: float):
+    """Router of a mixture of experts. logits fp32 [T, n]; scores are their
+    softmax; the choice adds `correction` [n] and is limited to the `keep`
+    best of `groups` equal groups of neighbouring outputs (a group's score
+    is its largest choice score). -> (chosen outputs int32 [T, top], their
+    uncorrected scores * scale fp32 [T, top])."""
+    if logits.is_cuda:
+        T = logits.shape[0]
+        idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+        wgt = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+        hip_seq().moe_route(idx, wgt, logits, correction, int(groups),
+                            int(keep), float(scale))
+        return idx, wgt
+    return seq_ref.moe_route(logits, correction, groups, keep, top, scale)
+
+
+def moe_dispatch(idx, n_out: int):
+    """-> (rank int32 [T, k]: how many earlier entries of idx chose the same
+    output, counts int32 [n_out])."""
+    if idx.is_cuda:
+        rank = torch.empty_like(idx)
+        counts = torch.empty(n_out, dtype=torch.int32, device=idx.device)
+        hip_seq().moe_dispatch(rank, counts, idx)
+        return rank, counts
+    return seq_ref.moe_dispatch(idx, n_out)
+
+
+def moe_gather(h, idx, rank, base, E: int, rows: int):
+    """xg [rows, W]: row base[e] + rank[t, j] holds h[t] for every choice
+    e = idx[t, j] < E (outputs >= E are identity experts and take no row).
+    Rows nobody owns are zero."""
+    if h.is_cuda:
+        xg = torch.zeros(rows, h.shape[1], dtype=h.dtype, device=h.device)
+        hip_seq().moe_gather(xg, h, idx, rank, base, int(E))
+        return xg
+    return seq_ref.moe_gather(h, idx, rank, base, E, rows)
+
+
+def moe_combine(y, h, idx, wgt, rank, base, E: int, shared, out_dtype):
+    """out[t] = sum_j wgt[t, j] * (y[base[e] + rank[t, j]] if e < E else
+    h[t]) (+ shared[t]), summed in fp32 in the order of j."""
+    if h.is_cuda:
+        out = torch.empty(h.shape, dtype=out_dtype, device=h.device)
+        hip_seq().moe_combine(out, y, h, idx, wgt, rank, base, int(E), shared)
+        return out
+    return seq_ref.moe_combine(y, h, idx, wgt, rank, base, E, shared,
+                               out_dtype)

@@ -303,7 +303,8 @@ def latent_append(cache, z, z_col, norm_w, slot_mapping, positions, freqs,
 
 
 def paged_attention_rows(q, off_q, H, kmaps, kcache, vcache, dv, positions, sb,
-                         scale, window):
+                         scale, window, keep_first=0, head_bias=None,
+                         sigmoid=False):
     """fp32 [T, H, kmaps, dv]; see ops.seq.paged_attention_rows."""
     P, G, ps, krow = kcache.shape
     dk = krow // kmaps
@@ -329,10 +330,16 @@ def paged_attention_rows(q, off_q, H, kmaps, kcache, vcache, dv, positions, sb,
         vv = vv.repeat_interleave(rep, 0)
         for t in range(start, start + n):
             i = pos[t]
-            lo = max(0, i + 1 - window) if window else 0
-            s = torch.einsum("hmd,hjmd->hmj", qq[t] * scale, kk[:, lo:i + 1])
-            out[t] = torch.einsum("hmj,hjd->hmd", torch.softmax(s, -1),
-                                  vv[:, lo:i + 1])
+            j = torch.arange(i + 1)
+            seen = ((i - j < window) | (j < keep_first)) if window else j >= 0
+            s = torch.einsum("hmd,hjmd->hmj", qq[t] * scale, kk[:, :i + 1])
+            if head_bias is not None:
+                s = s + head_bias.view(H, 1, 1)
+            if sigmoid:
+                wgt = torch.sigmoid(s) * seen
+            else:
+                wgt = torch.softmax(s.masked_fill(~seen, float("-inf")), -1)
+            out[t] = torch.einsum("hmj,hjd->hmd", wgt, vv[:, :i + 1])
     return out
 
 
@@ -396,4 +403,112 @@ def rglru_scan(u, gates, br, bi, lam, y, state, sb, decay, out_dtype):
             S = a[t] * S + b[t]
             out[t] = S * yy[t]
         state[slot] = S
+    return out.to(out_dtype)
+
+
+# -- sigmoid attention, minimal gated recurrence, routed experts ---------------
+def residual_conv(res, w, conv_state, sb, out_dtype):
+    """res + causal_conv(res) over the fp32 rows; see ops.seq.residual_conv."""
+    y = causal_conv(res, res.shape[1], w, None, False, conv_state, sb)
+    return (res + y).to(out_dtype)
+
+
+def headnorm_rope_append(proj, H, G, dk, dv, off_k, off_v, qw, kw, freqs,
+                         interleaved, eps, positions, kcache, vcache,
+                         slot_mapping):
+    T = proj.shape[0]
+    P, _g, ps, _d = kcache.shape
+
+    def normed(col, n, w):
+        x = proj[:, col:col + n * dk].float().view(T, n, dk)
+        x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w
+        if freqs is not None:
+            x = _rotate(x, positions, freqs, interleaved)
+        return x
+    q = normed(0, H, qw)
+    k = normed(off_k, G, kw).to(kcache.dtype)
+    proj[:, :H * dk] = q.reshape(T, H * dk).to(proj.dtype)
+    v = proj[:, off_v:off_v + G * dv].view(T, G, dv)
+    for t, slot in enumerate(slot_mapping.tolist()):
+        if slot < 0:
+            continue
+        kcache[slot // ps, :, slot % ps] = k[t]
+        vcache[slot // ps, :, slot % ps] = v[t]
+
+
+def mingru_scan(proj, C, state, sb, out_dtype):
+    """proj [T, 3C] = gate | candidate | output gate pre-activations."""
+    p = proj.float()
+    z = torch.sigmoid(p[:, :C])
+    keep = torch.sigmoid(-p[:, :C])
+    u = p[:, C:2 * C]
+    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    g = F.silu(p[:, 2 * C:3 * C])
+    out = torch.empty(p.shape[0], C, dtype=torch.float32)
+    for start, n, slot, pos0 in sb.spans():
+        if n == 0:
+            continue
+        S = state[slot].clone() if pos0 > 0 else torch.zeros(C)
+        for t in range(start, start + n):
+            S = keep[t] * S + z[t] * cand[t]
+            out[t] = S * g[t]
+        state[slot] = S
+    return out.to(out_dtype)
+
+
+def relu_squared(x):
+    y = x.float().clamp(min=0)
+    return (y * y).to(x.dtype)
+
+
+def moe_route(logits, correction, groups, keep, top, scale):
+    T, n = logits.shape
+    s = torch.softmax(logits.float(), -1)
+    choice = s + correction
+    if groups > 1:
+        size = n // groups
+        gs = choice.view(T, groups, size).max(-1).values
+        best = gs.topk(keep, -1).indices
+        ok = torch.zeros(T, groups, dtype=torch.bool)
+        ok.scatter_(1, best, True)
+        ok = ok[:, :, None].expand(T, groups, size).reshape(T, n)
+        choice = choice.masked_fill(~ok, float("-inf"))
+    idx = choice.topk(top, -1).indices
+    return idx.to(torch.int32), s.gather(1, idx) * scale
+
+
+def moe_dispatch(idx, n_out):
+    """rank [T, k]: how many earlier rows chose the same output;
+    counts [n_out]."""
+    T, k = idx.shape
+    flat = idx.reshape(-1).long()
+    onehot = F.one_hot(flat, n_out)
+    before = onehot.cumsum(0) - onehot
+    rank = before.gather(1, flat[:, None]).reshape(T, k)
+    return rank.to(torch.int32), onehot.sum(0).to(torch.int32)
+
+
+def moe_gather(h, idx, rank, base, E, rows):
+    xg = torch.zeros(rows, h.shape[1], dtype=h.dtype)
+    T, k = idx.shape
+    for t in range(T):
+        for j in range(k):
+            e = int(idx[t, j])
+            if e < E:
+                xg[int(base[e]) + int(rank[t, j])] = h[t]
+    return xg
+
+
+def moe_combine(y, h, idx, wgt, rank, base, E, shared, out_dtype):
+    T, k = idx.shape
+    out = torch.zeros(T, h.shape[1], dtype=torch.float32)
+    hf = h.float()
+    for t in range(T):
+        for j in range(k):
+            e = int(idx[t, j])
+            src = (y[int(base[e]) + int(rank[t, j])].float() if e < E
+                   else hf[t])
+            out[t] += wgt[t, j] * src
+    if shared is not None:
+        out += shared.float()
     return out.to(out_dtype)
