@@ -19,7 +19,11 @@
 // over the same values - the output is [T, H, kmaps, dv]), and a value row
 // stride of its own, so values may alias a prefix of the key rows (latent
 // attention, where the cached latent is both key part and value). The
-// output may be fp32 whatever the cache type.
+// output may be fp32 whatever the cache type. With a window, the first
+// `keep_first` keys of a sequence may stay visible whatever their distance;
+// a per-head constant may be added to the scaled scores; and the weights
+// may be plain sigmoids of the scores (not normalised over the keys)
+// instead of a softmax.
 #include "seq_common.h"
 
 namespace {
@@ -99,7 +103,8 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
     const int* __restrict__ seq_len, const float* __restrict__ r1,
     const float* __restrict__ r2, int H, int G, int dk, int dv, int ps,
     float scale, float temp_coef, int temp_every, int has_bias, int kmaps,
-    int vrow, int window) {
+    int vrow, int window, int keep_first, const float* __restrict__ head_bias,
+    int sigmoid) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // q [GS][dk]; merge [waves][GS][2 + dv]
   constexpr int VN = Vec16<T>::N;
@@ -127,11 +132,12 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
   }
   __syncthreads();
   const int* table = page_table + (int64_t)s * table_stride;
-  float b1[GS], b2[GS];
+  float b1[GS], b2[GS], hb[GS];
 #pragma unroll
   for (int a = 0; a < GS; a++) {
     b1[a] = has_bias ? r1[h0 + a] : 0.f;
     b2[a] = has_bias ? r2[h0 + a] : 0.f;
+    hb[a] = head_bias ? head_bias[h0 + a] : 0.f;
   }
   const int quad = lane >> 2, qq = lane & 3;
   const int nvec = dk / VN;  // 16-byte pieces of a key row (FAST)
@@ -149,7 +155,13 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
   const int ctx = pos + 1;
   const int jmin = window > 0 ? max(0, ctx - window) : 0;  // first visible key
   const int nchunks = (ctx + 63) >> 6;
-  for (int c = (jmin >> 6) + wave; c < nchunks; c += nwv) {
+  // chunks that hold kept first keys and lie wholly before the window's
+  // first chunk are walked first, then the window's chunks
+  const int c_lo = jmin >> 6;
+  const int nsink = (keep_first > 0 && jmin > 0)
+                        ? min((min(keep_first, jmin) + 63) >> 6, c_lo) : 0;
+  for (int vc = wave; vc < nsink + nchunks - c_lo; vc += nwv) {
+    const int c = vc < nsink ? vc : vc - nsink + c_lo;
     const int j0 = c << 6;
     // ---- scores: pass p covers keys j0 + 16 p + quad ----
     float sc[4][GS];
@@ -201,11 +213,19 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
         x += __shfl_xor(x, 1, 64);
         x += __shfl_xor(x, 2, 64);
         if (has_bias) x -= b1[a] * log1pf(b2[a] * (float)(pos - jc));
-        sc[p][a] = (j < ctx && j >= jmin) ? x : -INFINITY;
+        x += hb[a];
+        sc[p][a] = (j < ctx && (j >= jmin || j < keep_first)) ? x : -INFINITY;
       }
     }
     // ---- online softmax (every lane of a quad holds the same score) ----
     float pr[4][GS];
+    if (sigmoid) {
+      // unnormalised weights: a masked key (score -inf) weighs exactly 0
+#pragma unroll
+      for (int a = 0; a < GS; a++)
+#pragma unroll
+        for (int p = 0; p < 4; p++) pr[p][a] = sigmoid_f(sc[p][a]);
+    } else
 #pragma unroll
     for (int a = 0; a < GS; a++) {
       float mx = fmaxf(fmaxf(sc[0][a], sc[1][a]), fmaxf(sc[2][a], sc[3][a]));
@@ -309,6 +329,15 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
   }
   __syncthreads();
   for (int a = wave; a < GS; a += nwv) {  // wave a finishes head a
+    if (sigmoid) {  // plain sum of the waves' partial results
+      for (int ch = lane; ch < dv; ch += 64) {
+        float o = 0.f;
+        for (int w = 0; w < nwv; w++) o += mg[(w * GS + a) * MS + 2 + ch];
+        out[(((int64_t)t * H + h0 + a) * kmaps + map) * dv + ch] =
+            from_f<TO>(o);
+      }
+      continue;
+    }
     float mx = -INFINITY;
     for (int w = 0; w < nwv; w++) mx = fmaxf(mx, mg[(w * GS + a) * MS]);
     float lt = 0.f;
@@ -337,7 +366,8 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
                       c10::optional<torch::Tensor>& r1,
                       c10::optional<torch::Tensor>& r2, double scale,
                       double temp_coef, int64_t temp_every, int kmaps,
-                      int window) {
+                      int window, int keep_first,
+                      c10::optional<torch::Tensor>& head_bias, bool sigmoid) {
   const int T_ = out.size(0), H = out.size(1);
   const int G = kcache.size(1), ps = kcache.size(2);
   const int dk = kcache.size(3) / kmaps;
@@ -350,7 +380,7 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
   // window bounds the keys of a row, and the waves with them
   int NW = T_ * (H * kmaps / GS) <= 2048 ? 16 : 4;
   if (window > 0)
-    while (NW > 1 && (NW - 1) * 64 >= window + 63) NW >>= 1;
+    while (NW > 1 && (NW - 1) * 64 >= window + keep_first + 126) NW >>= 1;
   auto lds_bytes = [&](int gs, int nw) {
     return (size_t)(gs * dk + nw * gs * (2 + dv)) * sizeof(float);
   };
@@ -373,7 +403,8 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
       cptr<int>(tok_seq), cptr<int>(positions), cptr<int>(seq_len),         \
       r1 ? cptr<float>(*r1) : nullptr, r2 ? cptr<float>(*r2) : nullptr, H,  \
       G, dk, dv, ps, (float)scale, (float)temp_coef, (int)temp_every,       \
-      r1 ? 1 : 0, kmaps, vrow, window)
+      r1 ? 1 : 0, kmaps, vrow, window, keep_first,                          \
+      head_bias ? cptr<float>(*head_bias) : nullptr, sigmoid ? 1 : 0)
 #define LAUNCH_GS(GS_)                                                      \
   do {                                                                      \
     if (vec && small) LAUNCH_ATT(GS_, true, 2);                             \
@@ -429,9 +460,16 @@ void paged_attention_rows(torch::Tensor out, torch::Tensor proj, int64_t off_q,
                           c10::optional<torch::Tensor> r1,
                           c10::optional<torch::Tensor> r2, double scale,
                           double temp_coef, int64_t temp_every, int64_t kmaps,
-                          int64_t window) {
+                          int64_t window, int64_t keep_first,
+                          c10::optional<torch::Tensor> head_bias,
+                          bool sigmoid) {
   SEQ_CHECK(out.dim() == 4 && out.is_contiguous() && out.size(2) == kmaps,
             "attention out [T, H, maps, dv]");
+  SEQ_CHECK(keep_first >= 0, "kept first keys");
+  if (head_bias)
+    SEQ_CHECK(head_bias->scalar_type() == torch::kFloat &&
+                  head_bias->is_contiguous() &&
+                  head_bias->numel() == out.size(1), "head bias fp32 [H]");
   const int T_ = out.size(0), H = out.size(1), dv = out.size(3);
   const int G = kcache.size(1), krow = kcache.size(3);
   SEQ_CHECK(kmaps >= 1 && krow % kmaps == 0 && window >= 0, "key maps/window");
@@ -481,12 +519,13 @@ void paged_attention_rows(torch::Tensor out, torch::Tensor proj, int64_t off_q,
       launch_attention<T, float>(out, proj, off_q, kcache, vptr, dv, vrow,
                                  page_table, tok_seq, positions, seq_len, r1,
                                  r2, scale, temp_coef, temp_every, (int)kmaps,
-                                 (int)window);
+                                 (int)window, (int)keep_first, head_bias,
+                                 sigmoid);
     else
       launch_attention<T, T>(out, proj, off_q, kcache, vptr, dv, vrow,
                              page_table, tok_seq, positions, seq_len, r1, r2,
                              scale, temp_coef, temp_every, (int)kmaps,
-                             (int)window);
+                             (int)window, (int)keep_first, head_bias, sigmoid);
   });
 }
 
@@ -501,5 +540,5 @@ void biased_attention(torch::Tensor out, torch::Tensor proj, int64_t off_q,
                 out.scalar_type() == proj.scalar_type(), "attention out");
   paged_attention_rows(out.unsqueeze(2), proj, off_q, kcache, vcache,
                        page_table, tok_seq, positions, seq_len, r1, r2, scale,
-                       temp_coef, temp_every, 1, 0);
+                       temp_coef, temp_every, 1, 0, 0, c10::nullopt, false);
 }

@@ -3,7 +3,9 @@
 // products, everything between them is fp32. Options: a logarithmic
 // distance bias with a query temperature, a sliding window, several key
 // maps per kv head, values that alias the head of the key rows (latent
-// attention), fp32 output.
+// attention), fp32 output, kept first keys under a window, a per-head
+// constant on the scores, and plain sigmoid weights (not normalised over
+// the keys) in place of the softmax.
 //
 // A workgroup (4 waves) owns a tile of up to 64 consecutive rows of one
 // sequence and one (query head, key map); each wave owns 16 rows. Keys and
@@ -54,6 +56,7 @@ struct MfmaArgs {
   int H, G, dk, dv, ps;
   float scale, temp_coef; int temp_every, has_bias;
   int kmaps, krow, vrow, window;
+  int keep_first; const float* head_bias; int sigmoid;
   // HEADS mode: rows of a tile are heads of one decoded token
   const int* seq_len; int nsplit; float* partial;
 };
@@ -134,6 +137,12 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   }
   const float b1 = a.has_bias ? a.r1[h] : 0.f;
   const float b2 = a.has_bias ? a.r2[h] : 0.f;
+  float hb[4];  // constant added to the scaled scores of each row's head
+#pragma unroll
+  for (int r = 0; r < 4; r++)
+    hb[r] = !a.head_bias ? 0.f
+            : HEADS ? (ok_r[r] ? a.head_bias[h + wid * 16 + lg * 4 + r] : 0.f)
+                    : a.head_bias[h];
   // prompt rows are in order; the heads of a token share its position
   const int kv_end = a.positions[HEADS ? row0 : row0 + nrows - 1] + 1;
   // the first key any row of the tile sees
@@ -211,10 +220,21 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     }
   };
 
-  const int kstep = (HEADS ? a.nsplit : 1) * BN;
-  const int t_first = (kv_begin / BN + (HEADS ? (int)blockIdx.z : 0)) * BN;
-  if (t_first < kv_end) load_k(t_first, 0);
-  for (int t0 = t_first; t0 < kv_end; t0 += kstep) {
+  // key blocks: those that hold kept first keys and lie wholly before the
+  // window's first block, then the window's blocks
+  const int b_lo = kv_begin / BN;
+  const int nsink =
+      (a.keep_first > 0 && kv_begin > 0)
+          ? min((min(a.keep_first, kv_begin) + BN - 1) / BN, b_lo) : 0;
+  const int nvb = nsink + (kv_end + BN - 1) / BN - b_lo;
+  const int vstep = HEADS ? a.nsplit : 1;
+  auto block_t0 = [&](int vb) {
+    return (vb < nsink ? vb : vb - nsink + b_lo) * BN;
+  };
+  const int vb_first = HEADS ? (int)blockIdx.z : 0;
+  if (vb_first < nvb) load_k(block_t0(vb_first), 0);
+  for (int vb = vb_first; vb < nvb; vb += vstep) {
+    const int t0 = block_t0(vb);
     // ---- S = Q K^T over key-channel chunks: block n covers keys
     //      t0 + 16 n + lr
     f32x4_t s[4];
@@ -244,15 +264,30 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     }
     // ---- fp32: scale, penalty, mask, online softmax (rows 4 lg + r)
     float p[4][4];
+    if (a.sigmoid) {
+      // unnormalised weights: no running maximum, no rescaling
+#pragma unroll
+      for (int r = 0; r < 4; r++)
+#pragma unroll
+        for (int n = 0; n < 4; n++) {
+          const int j = t0 + n * 16 + lr;
+          const bool seen =
+              j <= pos_r[r] && (window == 0 || j > pos_r[r] - window ||
+                                j < a.keep_first);
+          p[n][r] = seen ? sigmoid_f(s[n][r] * qmul[r] + hb[r]) : 0.f;
+        }
+    } else
 #pragma unroll
     for (int r = 0; r < 4; r++) {
       float mt = -INFINITY;
 #pragma unroll
       for (int n = 0; n < 4; n++) {
         const int j = t0 + n * 16 + lr;
-        float x = s[n][r] * qmul[r];
+        float x = s[n][r] * qmul[r] + hb[r];
         if (a.has_bias) x -= b1 * log1pf(b2 * (float)max(pos_r[r] - j, 0));
-        const bool seen = j <= pos_r[r] && (window == 0 || j > pos_r[r] - window);
+        const bool seen =
+            j <= pos_r[r] && (window == 0 || j > pos_r[r] - window ||
+                              j < a.keep_first);
         x = seen ? x : -INFINITY;
         p[n][r] = x;
         mt = fmaxf(mt, x);
@@ -303,7 +338,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       if (vc) __syncthreads();  // the previous chunk's readers are done
       store_v(t0, vc);
       if (vc + 1 < NDCH) load_v(t0, vc + 1);
-      else if (t0 + kstep < kv_end) load_k(t0 + kstep, 0);
+      else if (vb + vstep < nvb) load_k(block_t0(vb + vstep), 0);
       __syncthreads();
       if (active)
 #pragma unroll
@@ -354,7 +389,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 #pragma unroll
   for (int r = 0; r < 4; r++) {
     if (!ok_r[r]) continue;
-    const float inv = 1.f / l[r];
+    const float inv = a.sigmoid ? 1.f : 1.f / l[r];
     TO* o = out + (((int64_t)(row0 + wid * 16 + lg * 4 + r) * H + h) * a.kmaps +
                    map) * dv;
 #pragma unroll
@@ -373,7 +408,7 @@ __global__ void merge_splits_kernel(float* __restrict__ out,
                                     const float* __restrict__ partial,
                                     const int* __restrict__ tok_seq,
                                     const int* __restrict__ seq_len,
-                                    int HM, int nsplit, int dv) {
+                                    int HM, int nsplit, int dv, int plain_sum) {
   const int t = blockIdx.x, hm = blockIdx.y;
   if (seq_len[tok_seq[t]] == 0) return;  // padding row
   const int rec = dv + 2;
@@ -390,8 +425,9 @@ __global__ void merge_splits_kernel(float* __restrict__ out,
   for (int z = 0; z < MAXSPLIT; z++) {
     w[z] = w[z] == -INFINITY ? 0.f : expf(w[z] - mx);
     if (z < nsplit) lt += w[z] * p[z * rec + 1];
+    if (plain_sum) w[z] = 1.f;  // unnormalised weights: the splits just add
   }
-  const float inv = 1.f / lt;
+  const float inv = plain_sum ? 1.f : 1.f / lt;
   for (int ch = threadIdx.x; ch < dv; ch += blockDim.x) {
     float o = 0.f;
 #pragma unroll
@@ -479,9 +515,16 @@ void paged_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
                           c10::optional<torch::Tensor> r1,
                           c10::optional<torch::Tensor> r2, double scale,
                           double temp_coef, int64_t temp_every, int64_t kmaps,
-                          int64_t window) {
+                          int64_t window, int64_t keep_first,
+                          c10::optional<torch::Tensor> head_bias,
+                          bool sigmoid) {
   SEQ_CHECK(out.dim() == 4 && out.is_contiguous() && out.size(2) == kmaps,
             "mfma attention out [T, H, maps, dv]");
+  SEQ_CHECK(keep_first >= 0, "kept first keys");
+  if (head_bias)
+    SEQ_CHECK(head_bias->scalar_type() == torch::kFloat &&
+                  head_bias->is_contiguous() &&
+                  head_bias->numel() == out.size(1), "head bias fp32 [H]");
   const int T_ = out.size(0), H = out.size(1), dv = out.size(3);
   const int G = kcache.size(1), ps = kcache.size(2), krow = kcache.size(3);
   SEQ_CHECK(kmaps >= 1 && krow % kmaps == 0 && window >= 0, "key maps/window");
@@ -546,6 +589,9 @@ void paged_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
   a.scale = (float)scale; a.temp_coef = (float)temp_coef;
   a.temp_every = (int)temp_every; a.has_bias = r1 ? 1 : 0;
   a.kmaps = (int)kmaps; a.krow = krow; a.vrow = vrow; a.window = (int)window;
+  a.keep_first = (int)keep_first;
+  a.head_bias = head_bias ? cptr<float>(*head_bias) : nullptr;
+  a.sigmoid = sigmoid ? 1 : 0;
   a.seq_len = nullptr; a.nsplit = 1; a.partial = nullptr;
   const int KC = pick_kc(dk), DN = pick_dn(dv);
   const dim3 grid(NT, H * kmaps);
@@ -565,10 +611,18 @@ void paged_attention_mfma_decode(torch::Tensor out, torch::Tensor partial,
                                  torch::Tensor page_table,
                                  torch::Tensor tok_seq, torch::Tensor positions,
                                  torch::Tensor seq_len, double scale,
-                                 int64_t kmaps, int64_t window) {
+                                 int64_t kmaps, int64_t window,
+                                 int64_t keep_first,
+                                 c10::optional<torch::Tensor> head_bias,
+                                 bool sigmoid) {
   SEQ_CHECK(out.dim() == 4 && out.is_contiguous() && out.size(2) == kmaps &&
                 out.scalar_type() == torch::kFloat,
             "mfma decode out [T, H, maps, dv] fp32");
+  SEQ_CHECK(keep_first >= 0, "kept first keys");
+  if (head_bias)
+    SEQ_CHECK(head_bias->scalar_type() == torch::kFloat &&
+                  head_bias->is_contiguous() &&
+                  head_bias->numel() == out.size(1), "head bias fp32 [H]");
   const int T_ = out.size(0), H = out.size(1), dv = out.size(3);
   const int G = kcache.size(1), ps = kcache.size(2), krow = kcache.size(3);
   SEQ_CHECK(kmaps >= 1 && krow % kmaps == 0 && window >= 0, "key maps/window");
@@ -624,6 +678,9 @@ void paged_attention_mfma_decode(torch::Tensor out, torch::Tensor partial,
   a.H = H; a.G = G; a.dk = dk; a.dv = dv; a.ps = ps;
   a.scale = (float)scale; a.temp_coef = 0.f; a.temp_every = 1; a.has_bias = 0;
   a.kmaps = (int)kmaps; a.krow = krow; a.vrow = vrow; a.window = (int)window;
+  a.keep_first = (int)keep_first;
+  a.head_bias = head_bias ? cptr<float>(*head_bias) : nullptr;
+  a.sigmoid = sigmoid ? 1 : 0;
   a.seq_len = cptr<int>(seq_len); a.nsplit = nsplit;
   a.partial = ptr<float>(partial);
   const int KC = pick_kc(dk), DN = pick_dn(dv);
@@ -636,7 +693,7 @@ void paged_attention_mfma_decode(torch::Tensor out, torch::Tensor partial,
                      dim3(dv <= 64 ? 64 : (dv <= 128 ? 128 : 256)), 0,
                      cur_stream(), ptr<float>(out), cptr<float>(partial),
                      cptr<int>(tok_seq), cptr<int>(seq_len), H * (int)kmaps,
-                     nsplit, dv);
+                     nsplit, dv, sigmoid ? 1 : 0);
 }
 
 void biased_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
@@ -650,5 +707,6 @@ void biased_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
   SEQ_CHECK(out.dim() == 3 && out.is_contiguous(), "mfma attention out");
   paged_attention_mfma(out.unsqueeze(2), proj, off_q, kcache, vcache,
                        page_table, tile_row0, tile_rows, max_tile_rows, tok_seq,
-                       positions, r1, r2, scale, temp_coef, temp_every, 1, 0);
+                       positions, r1, r2, scale, temp_coef, temp_every, 1, 0, 0,
+                       c10::nullopt, false);
 }

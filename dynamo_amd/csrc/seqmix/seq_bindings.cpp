@@ -1,6 +1,7 @@
 // Python bindings for the sequence-mixer kernels (dynamo_amd._hip_seq):
 // recurrent mixers (matrix-state and gated linear), paged attention over
-// rows (biased, windowed, multi-map, latent) and their row-wise companions. Built apart from dynamo_amd._hip so that a model which only
+// rows (biased, windowed, multi-map, latent, sigmoid-weighted), routed
+// experts and their row-wise companions. Built apart from dynamo_amd._hip so that a model which only
 // needs these compiles in seconds.
 #include <torch/extension.h>
 #include <pybind11/pybind11.h>
@@ -51,7 +52,9 @@ void paged_attention_rows(Tensor out, Tensor proj, int64_t off_q, Tensor kcache,
                           OptTensor vcache, Tensor page_table, Tensor tok_seq,
                           Tensor positions, Tensor seq_len, OptTensor r1,
                           OptTensor r2, double scale, double temp_coef,
-                          int64_t temp_every, int64_t kmaps, int64_t window);
+                          int64_t temp_every, int64_t kmaps, int64_t window,
+                          int64_t keep_first, OptTensor head_bias,
+                          bool sigmoid);
 void residual_layernorm(OptTensor out, Tensor res, OptTensor delta,
                         OptTensor post_w, double mult, OptTensor w, double eps);
 void xielu(Tensor out, Tensor x, Tensor pq);
@@ -75,7 +78,9 @@ void paged_attention_mfma(Tensor out, Tensor proj, int64_t off_q, Tensor kcache,
                           Tensor tile_rows, int64_t max_tile_rows,
                           Tensor tok_seq, Tensor positions, OptTensor r1,
                           OptTensor r2, double scale, double temp_coef,
-                          int64_t temp_every, int64_t kmaps, int64_t window);
+                          int64_t temp_every, int64_t kmaps, int64_t window,
+                          int64_t keep_first, OptTensor head_bias,
+                          bool sigmoid);
 void biased_attention_mfma(Tensor out, Tensor proj, int64_t off_q,
                            Tensor kcache, Tensor vcache, Tensor page_table,
                            Tensor tile_row0, Tensor tile_rows,
@@ -87,7 +92,28 @@ void paged_attention_mfma_decode(Tensor out, Tensor partial, Tensor proj,
                                  int64_t off_q, Tensor kcache, OptTensor vcache,
                                  Tensor page_table, Tensor tok_seq,
                                  Tensor positions, Tensor seq_len, double scale,
-                                 int64_t kmaps, int64_t window);
+                                 int64_t kmaps, int64_t window,
+                                 int64_t keep_first, OptTensor head_bias,
+                                 bool sigmoid);
+void residual_conv(Tensor out, Tensor x, Tensor w, Tensor conv_state,
+                   Tensor tok_seq, Tensor seq_start, Tensor seq_len,
+                   Tensor seq_slot, Tensor seq_pos0);
+void headnorm_rope_append(Tensor proj, int64_t H, int64_t G, int64_t dk,
+                          int64_t dv, int64_t off_k, int64_t off_v, Tensor qw,
+                          Tensor kw, OptTensor freqs, bool interleaved,
+                          double eps, Tensor positions, Tensor kcache,
+                          Tensor vcache, Tensor slot_mapping);
+void mingru_scan(Tensor out, Tensor proj, Tensor state, Tensor seq_start,
+                 Tensor seq_len, Tensor seq_slot, Tensor seq_pos0,
+                 int64_t max_len);
+void relu_squared(Tensor out, Tensor x);
+void moe_route(Tensor idx, Tensor wgt, Tensor logits, Tensor correction,
+               int64_t groups, int64_t keep, double scale);
+void moe_dispatch(Tensor rank, Tensor counts, Tensor idx);
+void moe_gather(Tensor xg, Tensor h, Tensor idx, Tensor rank, Tensor base,
+                int64_t E);
+void moe_combine(Tensor out, Tensor y, Tensor h, Tensor idx, Tensor wgt,
+                 Tensor rank, Tensor base, int64_t E, OptTensor shared);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "dynamo_amd sequence-mixer kernels (gfx950)";
@@ -118,4 +144,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("paged_attention_mfma_supported", &paged_attention_mfma_supported);
   m.def("paged_attention_mfma", &paged_attention_mfma);
   m.def("paged_attention_mfma_decode", &paged_attention_mfma_decode);
+  m.def("residual_conv", &residual_conv);
+  m.def("headnorm_rope_append", &headnorm_rope_append);
+  m.def("mingru_scan", &mingru_scan);
+  m.def("relu_squared", &relu_squared);
+  m.def("moe_route", &moe_route);
+  m.def("moe_dispatch", &moe_dispatch);
+  m.def("moe_gather", &moe_gather);
+  m.def("moe_combine", &moe_combine);
 }

@@ -69,6 +69,23 @@ DEVINL float logsigmoid_f(float x) {
   return fminf(x, 0.f) - log1pf(expf(-fabsf(x)));
 }
 
+// Rotation of one pair at angle pos * f, fp32 throughout. The frequency
+// comes as a float pair f = hi + lo; the rounding error of pos * hi is
+// recovered with an fma and, with pos * lo, applied as a first-order
+// correction to sin and cos, so the angle is good to about 1e-7 rad also
+// at positions in the tens of thousands (a plain fp32 product is off by
+// up to 6e-8 of the angle itself).
+DEVINL void rot_pair(float a, float b, float pos, float fhi, float flo,
+                     float& ra, float& rb) {
+  const float ang = pos * fhi;
+  const float rest = fmaf(pos, fhi, -ang) + pos * flo;
+  float sn, cs;
+  sincosf(ang, &sn, &cs);
+  const float s2 = fmaf(rest, cs, sn), c2 = fmaf(-rest, sn, cs);
+  ra = a * c2 - b * s2;
+  rb = b * c2 + a * s2;
+}
+
 #define SEQ_CHECK(cond, msg) TORCH_CHECK(cond, "seqmix: " msg)
 
 inline bool is_act(const torch::Tensor& t) {

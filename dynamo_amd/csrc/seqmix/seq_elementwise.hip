@@ -87,6 +87,44 @@ __global__ void causal_conv_kernel(
   }
 }
 
+// What a sublayer of a conv-fed layer reads: out = x + conv(x) over the fp32
+// residual rows x [T, W], a causal per-channel convolution whose last tap
+// weighs the current token. Rows before the portion come from the slot's
+// saved rows (zeros before position 0).
+template <typename TO>
+__global__ void residual_conv_kernel(
+    TO* __restrict__ out, const float* __restrict__ x,
+    const float* __restrict__ w, const float* __restrict__ conv_state,
+    const int* __restrict__ tok_seq, const int* __restrict__ seq_start,
+    const int* __restrict__ seq_slot, const int* __restrict__ seq_pos0,
+    int C, int taps) {
+  const int t = blockIdx.x;
+  const int s = tok_seq[t];
+  const int start = seq_start[s], pos0 = seq_pos0[s];
+  const float* st = conv_state + (int64_t)seq_slot[s] * (taps - 1) * C;
+  const int rel = t - start;  // rows of this portion before t
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    const float cur = x[(int64_t)t * C + c];
+    float acc = cur;
+    for (int j = 0; j < taps; j++) {
+      const int back = taps - 1 - j;  // how many tokens before t
+      float xv;
+      if (back == 0) {
+        xv = cur;
+      } else if (back <= rel) {
+        xv = x[(int64_t)(t - back) * C + c];
+      } else {
+        // state row i holds the input (taps-1-i) tokens before the portion
+        const int before = back - rel;  // 1..taps-1 tokens before the start
+        xv = (pos0 - before >= 0) ? st[(int64_t)(taps - 1 - before) * C + c]
+                                  : 0.f;
+      }
+      acc += w[c * taps + j] * xv;
+    }
+    out[(int64_t)t * C + c] = from_f<TO>(acc);
+  }
+}
+
 // After a step: the slot keeps the last taps-1 raw inputs of each sequence.
 template <typename T>
 __global__ void conv_state_update_kernel(
@@ -324,6 +362,44 @@ void causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
                          cptr<int>(seq_start), cptr<int>(seq_len),
                          cptr<int>(seq_slot), cptr<int>(seq_pos0), C, taps);
   });
+}
+
+void residual_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
+                   torch::Tensor conv_state, torch::Tensor tok_seq,
+                   torch::Tensor seq_start, torch::Tensor seq_len,
+                   torch::Tensor seq_slot, torch::Tensor seq_pos0) {
+  // x: fp32 [T, C]; out [T, C] = x + conv(x) in the activation type
+  const int T_ = x.size(0), C = w.size(0), taps = w.size(1);
+  const int B = seq_start.size(0);
+  SEQ_CHECK(x.dim() == 2 && x.scalar_type() == torch::kFloat &&
+                x.is_contiguous() && x.size(1) == C, "conv input fp32 [T, C]");
+  SEQ_CHECK(is_act(out) && out.is_contiguous() && out.size(0) == T_ &&
+                out.size(1) == C, "conv out");
+  SEQ_CHECK(w.scalar_type() == torch::kFloat && w.is_contiguous() && taps >= 1,
+            "conv w");
+  SEQ_CHECK(conv_state.scalar_type() == torch::kFloat &&
+                conv_state.is_contiguous() && conv_state.dim() == 3 &&
+                conv_state.size(1) == taps - 1 && conv_state.size(2) == C,
+            "conv state");
+  check_seq(tok_seq, T_, "tok_seq");
+  check_seq(seq_len, B, "seq_len");
+  check_seq(seq_slot, B, "seq_slot");
+  check_seq(seq_pos0, B, "seq_pos0");
+  if (T_ == 0) return;
+  DISPATCH_ACT(out, {
+    hipLaunchKernelGGL(residual_conv_kernel<T>, dim3(T_),
+                       dim3(std::min(256, row_block(C))), 0, cur_stream(),
+                       ptr<T>(out), cptr<float>(x), cptr<float>(w),
+                       cptr<float>(conv_state), cptr<int>(tok_seq),
+                       cptr<int>(seq_start), cptr<int>(seq_slot),
+                       cptr<int>(seq_pos0), C, taps);
+  });
+  if (taps > 1)
+    hipLaunchKernelGGL(conv_state_update_kernel<float>, dim3(B),
+                       dim3(row_block(C)), 0, cur_stream(),
+                       ptr<float>(conv_state), cptr<float>(x), C,
+                       cptr<int>(seq_start), cptr<int>(seq_len),
+                       cptr<int>(seq_slot), cptr<int>(seq_pos0), C, taps);
 }
 
 void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,
