@@ -56,12 +56,18 @@ def parse_args():
     p.add_argument("--mixer-compare", action="store_true",
                    help="instead of the flagship workload: prefill/decode "
                         "throughput of a layer-list design (see "
-                        "--mixer-model) beside Llama at equal sizes (1 GPU)")
+                        "--mixer-model) beside Llama or Mixtral at equal "
+                        "sizes (1 GPU)")
     p.add_argument("--mixer-model", default="bolatar",
-                   choices=["bolatar", "fironex"],
+                   choices=["bolatar", "fironex", "kefesun"],
                    help="which layer-list design --mixer-compare measures")
+    p.add_argument("--mixer-baseline", default=None,
+                   choices=["llama", "mixtral"],
+                   help="the model beside it (default: mixtral for a design "
+                        "with routed experts, else llama)")
     p.add_argument("--mixer-no-llama", action="store_true",
-                   help="--mixer-compare without the Llama runs (profiling)")
+                   help="--mixer-compare without the baseline runs "
+                        "(profiling)")
     p.add_argument("--mixer-sizes", default="small,medium",
                    help="comma list of benchmarks/mixer_compare.py SIZES")
     p.add_argument("--moe-ep", action="store_true",
@@ -467,7 +473,8 @@ def main():
             os.path.abspath(__file__)), "benchmarks"))
         import mixer_compare
         mixer_compare.run(args.mixer_sizes.split(","), device,
-                          args.mixer_model, not args.mixer_no_llama)
+                          args.mixer_model, not args.mixer_no_llama,
+                          args.mixer_baseline)
         return
     if world > 1:
         dist.init_process_group("nccl" if device.startswith("cuda") else "gloo")

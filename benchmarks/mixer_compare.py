@@ -1,10 +1,12 @@
-"""Prefill and decode throughput of a layer-list design (Bolatar or
-Fironex) beside the dense-attention Llama layout at equal width, depth,
-feed-forward size and vocabulary, random weights, one GPU, through the
-engine's own add_request/step loop (chunked prefill, then hipGraph decode).
+"""Prefill and decode throughput of a layer-list design (Bolatar, Fironex
+or Kefesun) beside the dense-attention Llama layout - or, for a design with
+routed experts, the Mixtral layout - at equal width, depth, feed-forward
+size and vocabulary, random weights, one GPU, through the engine's own
+add_request/step loop (chunked prefill, then hipGraph decode).
 
     python bench.py --mixer-compare [--mixer-sizes small,medium]
-                    [--mixer-model bolatar|fironex]
+                    [--mixer-model bolatar|fironex|kefesun]
+                    [--mixer-baseline llama|mixtral]
 
 Prints one JSON line: per size and model, prefill tokens/s (B prompts of
 ISL tokens until every request has its first token) and decode tokens/s
@@ -91,6 +93,46 @@ def fironex_config(width, layers, ff):
                        num_kv_heads=1, head_dim=1)
 
 
+def kefesun_config(width, layers, ff):
+    """Layer pattern: three sigmoid-attention layers (128-wide heads, four
+    query heads per kv head, a 1024-token window that keeps the first four
+    tokens) to one minimal gated recurrent unit of the model's width; every
+    layer with eight routed experts and two identity experts in two groups,
+    two per token, and a shared expert. A token's active feed-forward
+    weights equal those of a dense gated feed-forward of size ff."""
+    from dynamo_amd.engine.config import ModelConfig
+    H = width // 128
+    mlp = {"kind": "moe", "expert": {"ff": ff // 2},
+           "router": {"experts": 8, "identity": 2, "top": 2, "scale": 1.0,
+                      "groups": {"count": 2, "keep": 1}},
+           "shared": {"ff": ff // 2}}
+    attn = {"type": "attention", "mlp": mlp, "mixer": {
+        "heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128,
+        "scale": 128 ** -0.5, "mask": {"size": 1024, "keep_first": 4},
+        "rot": {"base": 10000.0, "dims": 64}}}
+    gru = {"type": "mingru", "mlp": mlp, "mixer": {"width": width}}
+    specs = [gru if i % 4 == 2 else attn for i in range(layers)]
+    return ModelConfig(name=f"kefesun-w{width}", arch="kefesun",
+                       hidden_size=width, vocab_size=VOCAB, max_position=8192,
+                       num_layers=layers, rms_eps=1e-6, embed_scale=1.0,
+                       conv_taps=4, tie_embeddings=True, norm="layernorm",
+                       layer_specs=specs, intermediate_size=0, num_q_heads=1,
+                       num_kv_heads=1, head_dim=1)
+
+
+def mixtral_config(width, layers, ff):
+    """Eight gated experts of size ff / 2, two per token: a token's active
+    feed-forward weights equal a dense gated feed-forward of size ff."""
+    from dynamo_amd.engine.config import ModelConfig
+    H = width // 128
+    return ModelConfig(name=f"mixtral-w{width}", arch="mixtral",
+                       hidden_size=width, intermediate_size=ff // 2,
+                       num_layers=layers, num_q_heads=H,
+                       num_kv_heads=max(1, H // 4), head_dim=128,
+                       vocab_size=VOCAB, max_position=8192, rope_theta=1e4,
+                       num_experts=8, num_experts_per_tok=2)
+
+
 def llama_config(width, layers, ff):
     from dynamo_amd.engine.config import ModelConfig
     H = width // 128
@@ -160,9 +202,13 @@ def measure(mc, s, device):
     return out
 
 
-def run(sizes, device="cuda:0", model="bolatar", with_llama=True):
+def run(sizes, device="cuda:0", model="bolatar", with_llama=True,
+        baseline=None):
     res = {}
-    make = {"bolatar": bolatar_config, "fironex": fironex_config}[model]
+    make = {"bolatar": bolatar_config, "fironex": fironex_config,
+            "kefesun": kefesun_config}[model]
+    baseline = baseline or ("mixtral" if model == "kefesun" else "llama")
+    base = {"llama": llama_config, "mixtral": mixtral_config}[baseline]
     for name in sizes:
         s = SIZES[name]
         args = (s["width"], s["layers"], s["ff"])
@@ -171,7 +217,7 @@ def run(sizes, device="cuda:0", model="bolatar", with_llama=True):
                                         "isl", "conc")},
             model: measure(make(*args), s, device)}
         if with_llama:
-            res[name]["llama"] = measure(llama_config(*args), s, device)
+            res[name][baseline] = measure(base(*args), s, device)
         print(f"# {name}: {json.dumps(res[name])}", flush=True)
     print(json.dumps({"metric": "mixer_compare", "dtype": "bf16",
                       "data": "synthetic", "sizes": res}), flush=True)

@@ -98,6 +98,9 @@ void paged_attention_mfma_decode(Tensor out, Tensor partial, Tensor proj,
 void residual_conv(Tensor out, Tensor x, Tensor w, Tensor conv_state,
                    Tensor tok_seq, Tensor seq_start, Tensor seq_len,
                    Tensor seq_slot, Tensor seq_pos0);
+bool join_conv_single(Tensor out, Tensor res, OptTensor delta, OptTensor post_w,
+                      double eps, Tensor w, Tensor conv_state, Tensor tok_seq,
+                      Tensor seq_len, Tensor seq_slot, Tensor seq_pos0);
 void headnorm_rope_append(Tensor proj, int64_t H, int64_t G, int64_t dk,
                           int64_t dv, int64_t off_k, int64_t off_v, Tensor qw,
                           Tensor kw, OptTensor freqs, bool interleaved,
@@ -107,8 +110,8 @@ void mingru_scan(Tensor out, Tensor proj, Tensor state, Tensor seq_start,
                  Tensor seq_len, Tensor seq_slot, Tensor seq_pos0,
                  int64_t max_len);
 void relu_squared(Tensor out, Tensor x);
-void moe_route(Tensor idx, Tensor wgt, Tensor logits, Tensor correction,
-               int64_t groups, int64_t keep, double scale);
+void moe_route(Tensor idx, Tensor wgt, Tensor logits, OptTensor router,
+               Tensor correction, int64_t groups, int64_t keep, double scale);
 void moe_dispatch(Tensor rank, Tensor counts, Tensor idx);
 void moe_gather(Tensor xg, Tensor h, Tensor idx, Tensor rank, Tensor base,
                 int64_t E);
@@ -145,6 +148,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("paged_attention_mfma", &paged_attention_mfma);
   m.def("paged_attention_mfma_decode", &paged_attention_mfma_decode);
   m.def("residual_conv", &residual_conv);
+  m.def("join_conv_single", &join_conv_single);
   m.def("headnorm_rope_append", &headnorm_rope_append);
   m.def("mingru_scan", &mingru_scan);
   m.def("relu_squared", &relu_squared);

@@ -91,37 +91,117 @@ __global__ void causal_conv_kernel(
 // residual rows x [T, W], a causal per-channel convolution whose last tap
 // weighs the current token. Rows before the portion come from the slot's
 // saved rows (zeros before position 0).
-template <typename TO>
+template <typename TO, int TAPS>
 __global__ void residual_conv_kernel(
     TO* __restrict__ out, const float* __restrict__ x,
     const float* __restrict__ w, const float* __restrict__ conv_state,
     const int* __restrict__ tok_seq, const int* __restrict__ seq_start,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_pos0,
-    int C, int taps) {
+    int C, int taps_rt) {
+  // one thread per (token, channel); TAPS > 0 fixes the tap count at
+  // compile time so that the loads of all taps issue together
+  const int taps = TAPS > 0 ? TAPS : taps_rt;
   const int t = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
   const int s = tok_seq[t];
   const int start = seq_start[s], pos0 = seq_pos0[s];
   const float* st = conv_state + (int64_t)seq_slot[s] * (taps - 1) * C;
   const int rel = t - start;  // rows of this portion before t
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
-    const float cur = x[(int64_t)t * C + c];
-    float acc = cur;
-    for (int j = 0; j < taps; j++) {
-      const int back = taps - 1 - j;  // how many tokens before t
-      float xv;
-      if (back == 0) {
-        xv = cur;
-      } else if (back <= rel) {
-        xv = x[(int64_t)(t - back) * C + c];
-      } else {
-        // state row i holds the input (taps-1-i) tokens before the portion
-        const int before = back - rel;  // 1..taps-1 tokens before the start
-        xv = (pos0 - before >= 0) ? st[(int64_t)(taps - 1 - before) * C + c]
-                                  : 0.f;
-      }
-      acc += w[c * taps + j] * xv;
+  const float cur = x[(int64_t)t * C + c];
+  float acc = cur;
+#pragma unroll
+  for (int j = 0; j < taps; j++) {
+    const int back = taps - 1 - j;  // how many tokens before t
+    float xv;
+    if (back == 0) {
+      xv = cur;
+    } else if (back <= rel) {
+      xv = x[(int64_t)(t - back) * C + c];
+    } else {
+      // state row i holds the input (taps-1-i) tokens before the portion
+      const int before = back - rel;  // 1..taps-1 tokens before the start
+      xv = (pos0 - before >= 0) ? st[(int64_t)(taps - 1 - before) * C + c]
+                                : 0.f;
     }
-    out[(int64_t)t * C + c] = from_f<TO>(acc);
+    acc += w[c * taps + j] * xv;
+  }
+  out[(int64_t)t * C + c] = from_f<TO>(acc);
+}
+
+// Decoded tokens (every sequence brings one row): the waiting sublayer
+// output joins the residual stream and the next sublayer's input is formed
+// in one pass over the row,
+//   x += LN(delta) * post_w;  out = x + conv(x);  slot rows <- shifted + x,
+// with LN the weight-only layer norm (two passes over registers) and the
+// convolution reading the slot's saved rows. A thread owns NI channels of
+// its row, so every state entry is read and written by one thread only.
+// Padding rows (seq_len 0) leave the slot alone.
+template <typename T, int TAPS, int NI>
+__global__ void join_conv_single_kernel(
+    T* __restrict__ out, float* __restrict__ res, const T* __restrict__ delta,
+    const float* __restrict__ post_w, float eps, const float* __restrict__ cw,
+    float* __restrict__ conv_state, const int* __restrict__ tok_seq,
+    const int* __restrict__ seq_len, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_pos0, int W) {
+  __shared__ float scratch[16];
+  constexpr int K = TAPS - 1;
+  const int t = blockIdx.x;
+  const int s = tok_seq[t];
+  const bool live = seq_len[s] == 1;
+  const int pos0 = seq_pos0[s];
+  float* st = conv_state + (int64_t)seq_slot[s] * K * W;
+  float* r = res + (int64_t)t * W;
+  float x[NI], hist[NI][K > 0 ? K : 1];
+#pragma unroll
+  for (int k = 0; k < NI; k++) {
+    const int i = threadIdx.x + k * blockDim.x;
+    x[k] = i < W ? r[i] : 0.f;
+#pragma unroll
+    for (int j = 0; j < K; j++)  // row j: the input K - j tokens back
+      hist[k][j] = (i < W && pos0 - (K - j) >= 0) ? st[(int64_t)j * W + i] : 0.f;
+  }
+  if (delta) {
+    const T* dl = delta + (int64_t)t * W;
+    float d[NI];
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < NI; k++) {
+      const int i = threadIdx.x + k * blockDim.x;
+      d[k] = i < W ? to_f(dl[i]) : 0.f;
+      sum += d[k];
+    }
+    const float mean = block_sum(sum, scratch) / (float)W;
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < NI; k++) {
+      const int i = threadIdx.x + k * blockDim.x;
+      const float c = i < W ? d[k] - mean : 0.f;
+      ss += c * c;
+    }
+    const float inv = 1.f / sqrtf(block_sum(ss, scratch) / (float)W + eps);
+#pragma unroll
+    for (int k = 0; k < NI; k++) {
+      const int i = threadIdx.x + k * blockDim.x;
+      if (i < W) {
+        x[k] += (d[k] - mean) * inv * post_w[i];
+        r[i] = x[k];
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < NI; k++) {
+    const int i = threadIdx.x + k * blockDim.x;
+    if (i >= W) continue;
+    float acc = x[k] + cw[i * TAPS + K] * x[k];
+#pragma unroll
+    for (int j = 0; j < K; j++) acc += cw[i * TAPS + j] * hist[k][j];
+    out[(int64_t)t * W + i] = from_f<T>(acc);
+    if (live) {
+#pragma unroll
+      for (int j = 0; j + 1 < K; j++) st[(int64_t)j * W + i] = hist[k][j + 1];
+      if (K > 0) st[(int64_t)(K - 1) * W + i] = x[k];
+    }
   }
 }
 
@@ -386,20 +466,88 @@ void residual_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
   check_seq(seq_slot, B, "seq_slot");
   check_seq(seq_pos0, B, "seq_pos0");
   if (T_ == 0) return;
+  const int threads = std::min(256, row_block(C));
+  const dim3 grid(T_, (C + threads - 1) / threads);
+#define CONV_LAUNCH(TAPS_)                                                   \
+  hipLaunchKernelGGL((residual_conv_kernel<T, TAPS_>), grid, dim3(threads),  \
+                     0, cur_stream(), ptr<T>(out), cptr<float>(x),           \
+                     cptr<float>(w), cptr<float>(conv_state),                \
+                     cptr<int>(tok_seq), cptr<int>(seq_start),               \
+                     cptr<int>(seq_slot), cptr<int>(seq_pos0), C, taps)
   DISPATCH_ACT(out, {
-    hipLaunchKernelGGL(residual_conv_kernel<T>, dim3(T_),
-                       dim3(std::min(256, row_block(C))), 0, cur_stream(),
-                       ptr<T>(out), cptr<float>(x), cptr<float>(w),
-                       cptr<float>(conv_state), cptr<int>(tok_seq),
-                       cptr<int>(seq_start), cptr<int>(seq_slot),
-                       cptr<int>(seq_pos0), C, taps);
+    if (taps == 4) CONV_LAUNCH(4);
+    else if (taps == 2) CONV_LAUNCH(2);
+    else if (taps == 3) CONV_LAUNCH(3);
+    else CONV_LAUNCH(0);
   });
+#undef CONV_LAUNCH
   if (taps > 1)
     hipLaunchKernelGGL(conv_state_update_kernel<float>, dim3(B),
                        dim3(row_block(C)), 0, cur_stream(),
                        ptr<float>(conv_state), cptr<float>(x), C,
                        cptr<int>(seq_start), cptr<int>(seq_len),
                        cptr<int>(seq_slot), cptr<int>(seq_pos0), C, taps);
+}
+
+// One row per sequence (decoded tokens). delta/post_w absent: the stream is
+// taken as it is. Returns false (nothing done) for sizes the fused kernel
+// is not built for; the caller then takes the separate kernels.
+bool join_conv_single(torch::Tensor out, torch::Tensor res,
+                      c10::optional<torch::Tensor> delta,
+                      c10::optional<torch::Tensor> post_w, double eps,
+                      torch::Tensor w, torch::Tensor conv_state,
+                      torch::Tensor tok_seq, torch::Tensor seq_len,
+                      torch::Tensor seq_slot, torch::Tensor seq_pos0) {
+  const int T_ = res.size(0), W = res.size(1), taps = w.size(1);
+  const int B = seq_len.size(0);
+  if (taps < 1 || taps > 4 || W > 8192) return false;
+  SEQ_CHECK(res.dim() == 2 && res.scalar_type() == torch::kFloat &&
+                res.is_contiguous(), "res");
+  SEQ_CHECK(is_act(out) && out.is_contiguous() && out.size(0) == T_ &&
+                out.size(1) == W, "conv out");
+  SEQ_CHECK(delta.has_value() == post_w.has_value(), "delta and its weight");
+  if (delta)
+    SEQ_CHECK(delta->is_contiguous() && delta->size(0) == T_ &&
+                  delta->size(1) == W &&
+                  delta->scalar_type() == out.scalar_type() &&
+                  post_w->scalar_type() == torch::kFloat &&
+                  post_w->is_contiguous() && post_w->numel() == W, "delta");
+  SEQ_CHECK(w.scalar_type() == torch::kFloat && w.is_contiguous() &&
+                w.size(0) == W, "conv w");
+  SEQ_CHECK(conv_state.scalar_type() == torch::kFloat &&
+                conv_state.is_contiguous() && conv_state.dim() == 3 &&
+                conv_state.size(1) == taps - 1 && conv_state.size(2) == W,
+            "conv state");
+  check_seq(tok_seq, T_, "tok_seq");
+  check_seq(seq_len, B, "seq_len");
+  check_seq(seq_slot, B, "seq_slot");
+  check_seq(seq_pos0, B, "seq_pos0");
+  if (T_ == 0) return true;
+  const int threads = std::min(1024, row_block((W + 3) / 4));
+  const int ni = (W + threads - 1) / threads;
+#define JC_LAUNCH(TAPS_, NI_)                                                \
+  hipLaunchKernelGGL((join_conv_single_kernel<T, TAPS_, NI_>), dim3(T_),     \
+                     dim3(threads), 0, cur_stream(), ptr<T>(out),            \
+                     ptr<float>(res),                                        \
+                     delta ? cptr<T>(*delta) : (const T*)nullptr,            \
+                     post_w ? cptr<float>(*post_w) : (const float*)nullptr,  \
+                     (float)eps, cptr<float>(w), ptr<float>(conv_state),     \
+                     cptr<int>(tok_seq), cptr<int>(seq_len),                 \
+                     cptr<int>(seq_slot), cptr<int>(seq_pos0), W)
+#define JC_TAPS(NI_)                                                         \
+  do {                                                                       \
+    if (taps == 4) JC_LAUNCH(4, NI_);                                        \
+    else if (taps == 3) JC_LAUNCH(3, NI_);                                   \
+    else if (taps == 2) JC_LAUNCH(2, NI_);                                   \
+    else JC_LAUNCH(1, NI_);                                                  \
+  } while (0)
+  DISPATCH_ACT(out, {
+    if (ni <= 4) JC_TAPS(4);
+    else JC_TAPS(8);
+  });
+#undef JC_TAPS
+#undef JC_LAUNCH
+  return true;
 }
 
 void causal_conv_silu(torch::Tensor out, torch::Tensor x, torch::Tensor w,

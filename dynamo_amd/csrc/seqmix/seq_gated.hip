@@ -219,9 +219,15 @@ DEVINL void wave_argmax(float& v, int& i) {
 // are out of the running; the `top` largest remaining choices are taken in
 // falling order and weigh in with s * scale.
 // LDS per wave: s [n], choice [n], group score [groups].
+// The logits are given (fp32 [T, n]), or - for few rows - formed here as
+// the fp32 products of the token's input h [W] (activation type) with the
+// router's fp32 rows [n, W], eight outputs at a time.
+template <typename T>
 __global__ __launch_bounds__(256) void moe_route_kernel(
     int* __restrict__ idx, float* __restrict__ wgt,
-    const float* __restrict__ logits, const float* __restrict__ correction,
+    const float* __restrict__ logits, const T* __restrict__ h,
+    const float* __restrict__ router, int W,
+    const float* __restrict__ correction,
     int T_, int n, int groups, int keep, int top, float scale) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -230,7 +236,29 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
   float* sc = lds + wave * (2 * n + groups);
   float* ch = sc + n;
   float* gs = ch + n;
-  const float* z = logits + (int64_t)t * n;
+  if (logits) {
+    for (int i = lane; i < n; i += 64) ch[i] = logits[(int64_t)t * n + i];
+  } else {
+    const T* hr = h + (int64_t)t * W;
+    for (int i0 = 0; i0 < n; i0 += 8) {
+      float acc[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++) acc[u] = 0.f;
+      for (int c = lane; c < W; c += 64) {
+        const float hv = to_f(hr[c]);
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+          acc[u] += hv * router[(int64_t)min(i0 + u, n - 1) * W + c];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const float v = wave_sum(acc[u]);
+        if (lane == 0 && i0 + u < n) ch[i0 + u] = v;
+      }
+    }
+  }
+  wave_sync();
+  const float* z = ch;  // raw logits, replaced by the choice scores below
   float mx = -INFINITY;
   for (int i = lane; i < n; i += 64) mx = fmaxf(mx, z[i]);
   mx = wave_max(mx);
@@ -497,12 +525,22 @@ void relu_squared(torch::Tensor out, torch::Tensor x) {
   });
 }
 
+// `logits` fp32 [T, n], or - with `router` fp32 [n, W] given - the router's
+// input rows h [T, W] in the activation type.
 void moe_route(torch::Tensor idx, torch::Tensor wgt, torch::Tensor logits,
-               torch::Tensor correction, int64_t groups, int64_t keep,
-               double scale) {
-  const int T_ = logits.size(0), n = logits.size(1), top = idx.size(1);
-  SEQ_CHECK(logits.dim() == 2 && logits.scalar_type() == torch::kFloat &&
-                logits.is_contiguous(), "router logits fp32 [T, n]");
+               c10::optional<torch::Tensor> router, torch::Tensor correction,
+               int64_t groups, int64_t keep, double scale) {
+  const int T_ = logits.size(0), top = idx.size(1);
+  const int n = router ? router->size(0) : logits.size(1);
+  if (router) {
+    SEQ_CHECK(is_act(logits) && logits.dim() == 2 && logits.is_contiguous() &&
+                  router->scalar_type() == torch::kFloat &&
+                  router->is_contiguous() && router->dim() == 2 &&
+                  router->size(1) == logits.size(1), "router input and rows");
+  } else {
+    SEQ_CHECK(logits.dim() == 2 && logits.scalar_type() == torch::kFloat &&
+                  logits.is_contiguous(), "router logits fp32 [T, n]");
+  }
   SEQ_CHECK(correction.scalar_type() == torch::kFloat &&
                 correction.is_contiguous() && correction.numel() == n,
             "router correction");
@@ -516,10 +554,20 @@ void moe_route(torch::Tensor idx, torch::Tensor wgt, torch::Tensor logits,
   const size_t lds = 4 * (2 * (size_t)n + groups) * sizeof(float);
   SEQ_CHECK(lds <= 64 * 1024, "too many router outputs");
   if (T_ == 0) return;
-  hipLaunchKernelGGL(moe_route_kernel, dim3((T_ + 3) / 4), dim3(256), lds,
-                     cur_stream(), ptr<int>(idx), ptr<float>(wgt),
-                     cptr<float>(logits), cptr<float>(correction), T_, n,
-                     (int)groups, (int)keep, top, (float)scale);
+  if (router) {
+    DISPATCH_ACT(logits, hipLaunchKernelGGL(
+        moe_route_kernel<T>, dim3((T_ + 3) / 4), dim3(256), lds, cur_stream(),
+        ptr<int>(idx), ptr<float>(wgt), (const float*)nullptr,
+        cptr<T>(logits), cptr<float>(*router), (int)logits.size(1),
+        cptr<float>(correction), T_, n, (int)groups, (int)keep, top,
+        (float)scale););
+  } else {
+    hipLaunchKernelGGL(moe_route_kernel<float>, dim3((T_ + 3) / 4), dim3(256),
+                       lds, cur_stream(), ptr<int>(idx), ptr<float>(wgt),
+                       cptr<float>(logits), (const float*)nullptr,
+                       (const float*)nullptr, 0, cptr<float>(correction), T_,
+                       n, (int)groups, (int)keep, top, (float)scale);
+  }
 }
 
 void moe_dispatch(torch::Tensor rank, torch::Tensor counts, torch::Tensor idx) {

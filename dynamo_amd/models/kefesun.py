@@ -164,25 +164,28 @@ class KefesunForCausalLM(torch.nn.Module):
             sops.residual_layernorm(x, delta, w, 1.0, None, self.eps,
                                     self.dtype)
 
-        def read(conv_w, tail):    # what a sublayer reads: x + conv(x)
+        def read(last, conv_w, tail):
+            """The waiting sublayer output joins the stream; returns what
+            the next sublayer reads: x + conv(x)."""
+            delta, post = last if last is not None else (None, None)
             if conv_w is None:
+                if delta is not None:
+                    join(delta, post)
                 return x.to(self.dtype)
-            return sops.residual_conv(x, conv_w, tail, sb, self.dtype)
-        last = None     # the last sublayer's output joins in the final norm
+            return sops.join_conv(x, delta, post, self.eps, conv_w, tail, sb,
+                                  self.dtype)
+        last = None     # (sublayer output, its norm weight) not yet joined
         for i, layer in enumerate(self.layers):
-            if last is not None:
-                join(*last)
             st = states.layer(i)
             nconv = self._nconv(layer)
-            h = read(layer.canon1, st[0] if nconv else None)
+            h = read(last, layer.canon1, st[0] if nconv else None)
             shape = layer.mixer.kv_shape()
             ctx = MixContext(sb, meta.positions, meta.slot_mapping, st[nconv:],
                              kv_pool.kcache(i) if shape else None,
                              kv_pool.vcache(i) if shape else None)
             last = (layer.mixer.forward(h, ctx), layer.norm1)
             if layer.mlp is not None:
-                join(*last)
-                h = read(layer.canon2, st[1] if nconv else None)
+                h = read(last, layer.canon2, st[1] if nconv else None)
                 last = (layer.mlp.forward(h), layer.norm2)
             if tap is not None:     # residual after the layer (diagnostics)
                 join(*last)

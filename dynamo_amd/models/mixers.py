@@ -722,9 +722,9 @@ class RoutedExperts(torch.nn.Module):
 
     def forward(self, h):
         T, E = h.shape[0], self.E
-        logits = F.linear(h.float(), self.router)
-        idx, wgt = sops.moe_route(logits, self.correction, self.groups,
-                                  self.keep, self.top, self.scale)
+        idx, wgt = sops.moe_route_rows(h, self.router, self.correction,
+                                       self.groups, self.keep, self.top,
+                                       self.scale)
         rank, counts = sops.moe_dispatch(idx, self.n)
         if T <= self.PADDED_MAX_ROWS:
             # every expert gets a block of T rows: static shapes, no host read

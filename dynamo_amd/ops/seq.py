@@ -413,6 +413,24 @@ def residual_conv(res, w, conv_state, sb: SeqBatch, out_dtype):
     return seq_ref.residual_conv(res, w, conv_state, sb, out_dtype)
 
 
+def join_conv(res, delta, post_w, eps: float, w, conv_state, sb: SeqBatch,
+              out_dtype):
+    """The step between two sublayers of a conv-fed layer: the waiting
+    sublayer output joins the stream, res += LN(delta) * post_w (weight-only
+    layer norm; skipped without delta), and the next sublayer's input
+    res + conv(res) is returned (see residual_conv). When every row is a
+    decoded token both happen in one kernel."""
+    if res.is_cuda and sb.num_decode >= res.shape[0] and w.shape[1] <= 4:
+        out = torch.empty(res.shape, dtype=out_dtype, device=res.device)
+        if hip_seq().join_conv_single(out, res, delta, post_w, float(eps), w,
+                                      conv_state, sb.tok_seq, sb.seq_len,
+                                      sb.seq_slot, sb.seq_pos0):
+            return out
+    if delta is not None:
+        residual_layernorm(res, delta, post_w, 1.0, None, eps, out_dtype)
+    return residual_conv(res, w, conv_state, sb, out_dtype)
+
+
 def headnorm_rope_append(proj, H: int, G: int, dk: int, dv: int, off_k: int,
                          off_v: int, qw, kw, freqs, interleaved: bool,
                          eps: float, positions, kcache, vcache, slot_mapping):
@@ -474,10 +492,26 @@ def moe_route(logits, correction, groups: int, keep: int, top: int,
         T = logits.shape[0]
         idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
         wgt = torch.empty(T, top, dtype=torch.float32, device=logits.device)
-        hip_seq().moe_route(idx, wgt, logits, correction, int(groups),
+        hip_seq().moe_route(idx, wgt, logits, None, correction, int(groups),
                             int(keep), float(scale))
         return idx, wgt
     return seq_ref.moe_route(logits, correction, groups, keep, top, scale)
+
+
+def moe_route_rows(h, router, correction, groups: int, keep: int, top: int,
+                   scale: float):
+    """moe_route of the fp32 logits h @ router^T (h [T, W] in the activation
+    type, router fp32 [n, W]). Few rows with few router outputs form their
+    logits inside the routing kernel."""
+    T, n = h.shape[0], router.shape[0]
+    if h.is_cuda and T <= 256 and n <= 64:
+        idx = torch.empty(T, top, dtype=torch.int32, device=h.device)
+        wgt = torch.empty(T, top, dtype=torch.float32, device=h.device)
+        hip_seq().moe_route(idx, wgt, h, router, correction, int(groups),
+                            int(keep), float(scale))
+        return idx, wgt
+    logits = torch.nn.functional.linear(h.float(), router)
+    return moe_route(logits, correction, groups, keep, top, scale)
 
 
 def moe_dispatch(idx, n_out: int):
@@ -493,10 +527,11 @@ def moe_dispatch(idx, n_out: int):
 
 def moe_gather(h, idx, rank, base, E: int, rows: int):
     """xg [rows, W]: row base[e] + rank[t, j] holds h[t] for every choice
-    e = idx[t, j] < E (outputs >= E are identity experts and take no row).
-    Rows nobody owns are zero."""
+    e = idx[t, j] < E (outputs >= E are identity experts and take no row)."""
     if h.is_cuda:
-        xg = torch.zeros(rows, h.shape[1], dtype=h.dtype, device=h.device)
+        # rows nobody owns stay as they are: nothing reads what the experts
+        # make of them
+        xg = torch.empty(rows, h.shape[1], dtype=h.dtype, device=h.device)
         hip_seq().moe_gather(xg, h, idx, rank, base, int(E))
         return xg
     return seq_ref.moe_gather(h, idx, rank, base, E, rows)

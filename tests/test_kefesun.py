@@ -142,6 +142,50 @@ def test_ops_carry_state_across_portions(device, taps):
         assert torch.allclose(y0, y1, atol=1e-5)
 
 
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("taps,W", [(1, 20), (2, 33), (4, 20), (5, 20),
+                                    (3, 700), (4, 4100)])
+def test_join_and_convolution_of_decoded_rows(device, taps, W):
+    """Rows that are all decoded tokens take the fused step (the waiting
+    output is normed and added, the convolution reads and advances the
+    slot's rows): three sequences at different positions, one of them at
+    its second token, against the whole-sequence computation."""
+    from dynamo_amd.ops import seq as sops
+    g = torch.Generator().manual_seed(taps * W)
+    lens = [9, 2, 5]
+    xs = [torch.randn(n, W, generator=g) for n in lens]      # streams
+    ds = [torch.randn(n, W, generator=g) for n in lens]      # waiting outputs
+    cw = torch.randn(W, taps, generator=g)
+    pw = torch.rand(W, generator=g) + 0.5
+    want = []
+    for x, d in zip(xs, ds):
+        y = x.double() + oracle.layer_norm(d.double(), pw, 1e-5)
+        want.append(y + oracle.time_conv(y, cw))
+    cs = torch.full((4, taps - 1, W), 7.0, device=device)    # dirty slots
+    slots = [2, 0, 3]
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=device)  # noqa: E731
+    # all but the last token of each sequence as a prompt portion
+    for k, n in enumerate(lens):
+        sb = _span(n - 1, slots[k], 0, device)
+        sops.join_conv(xs[k][:n - 1].clone().to(device),
+                       ds[k][:n - 1].to(device), pw.to(device), 1e-5,
+                       cw.to(device), cs, sb, torch.float32)
+    # the last tokens together, as decoded rows
+    res = torch.stack([x[-1] for x in xs]).to(device)
+    delta = torch.stack([d[-1] for d in ds]).to(device)
+    sb = sops.SeqBatch(i32([0, 1, 2]), i32([0, 1, 2]), i32([1, 1, 1]),
+                       i32(slots), i32([n - 1 for n in lens]), num_decode=3,
+                       host=[(k, 1, slots[k], lens[k] - 1) for k in range(3)])
+    got = sops.join_conv(res, delta, pw.to(device), 1e-5, cw.to(device), cs,
+                         sb, torch.float32).cpu()
+    for k in range(3):
+        assert torch.allclose(got[k].double(), want[k][-1], atol=1e-4)
+        y = xs[k].double() + oracle.layer_norm(ds[k].double(), pw, 1e-5)
+        if taps > 1:      # the slot now ends with this token's stream row
+            assert torch.allclose(cs[slots[k], -1].cpu().double(), y[-1],
+                                  atol=1e-5)
+
+
 # -- the router -----------------------------------------------------------------
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("n,groups,keep,top", [(6, 3, 2, 3), (8, 1, 1, 2),
@@ -170,6 +214,20 @@ def test_router_against_oracle(device, n, groups, keep, top):
     worder = want_idx.argsort(-1)
     assert torch.allclose(wgt.cpu().double().gather(1, order),
                           want_w.gather(1, worder), atol=1e-6)
+    # the same from the router's input rows (few rows: logits formed in
+    # the routing kernel), fp32 and bf16 rows
+    for dt in (torch.float32, torch.bfloat16):
+        hh = h.to(dt)
+        want_idx2, want_w2 = oracle.route(hh.double(), Wt, "p.", r)
+        idx2, wgt2 = sops.moe_route_rows(
+            hh.to(device), Wt["p.router"].to(device),
+            Wt["p.correction"].to(device), groups, keep, top, 2.5)
+        same = (idx2.cpu().long().sort(-1).values
+                == want_idx2.sort(-1).values).all(-1)
+        assert float(same.float().mean()) > 0.9      # near-ties may flip
+        o2, w2 = idx2.cpu().long().argsort(-1), want_idx2.argsort(-1)
+        assert torch.allclose(wgt2.cpu().double().gather(1, o2)[same],
+                              want_w2.gather(1, w2)[same], atol=1e-5)
     if groups > 1 and keep < groups:
         s = torch.softmax(h @ Wt["p.router"].double().t(), -1)
         choice = s + Wt["p.correction"].double()
