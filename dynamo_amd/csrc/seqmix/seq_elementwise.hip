@@ -152,14 +152,19 @@ __global__ void join_conv_single_kernel(
   const int pos0 = seq_pos0[s];
   float* st = conv_state + (int64_t)seq_slot[s] * K * W;
   float* r = res + (int64_t)t * W;
-  float x[NI], hist[NI][K > 0 ? K : 1];
+  float x[NI], hist[NI][K > 0 ? K : 1], wt[NI][TAPS], pw[NI];
+  // everything the row needs is requested before the first reduction
 #pragma unroll
   for (int k = 0; k < NI; k++) {
     const int i = threadIdx.x + k * blockDim.x;
+    const int ic = min(i, W - 1);
     x[k] = i < W ? r[i] : 0.f;
 #pragma unroll
     for (int j = 0; j < K; j++)  // row j: the input K - j tokens back
       hist[k][j] = (i < W && pos0 - (K - j) >= 0) ? st[(int64_t)j * W + i] : 0.f;
+#pragma unroll
+    for (int j = 0; j < TAPS; j++) wt[k][j] = cw[ic * TAPS + j];
+    pw[k] = post_w ? post_w[ic] : 0.f;
   }
   if (delta) {
     const T* dl = delta + (int64_t)t * W;
@@ -184,7 +189,7 @@ __global__ void join_conv_single_kernel(
     for (int k = 0; k < NI; k++) {
       const int i = threadIdx.x + k * blockDim.x;
       if (i < W) {
-        x[k] += (d[k] - mean) * inv * post_w[i];
+        x[k] += (d[k] - mean) * inv * pw[k];
         r[i] = x[k];
       }
     }
@@ -193,9 +198,9 @@ __global__ void join_conv_single_kernel(
   for (int k = 0; k < NI; k++) {
     const int i = threadIdx.x + k * blockDim.x;
     if (i >= W) continue;
-    float acc = x[k] + cw[i * TAPS + K] * x[k];
+    float acc = x[k] + wt[k][K] * x[k];
 #pragma unroll
-    for (int j = 0; j < K; j++) acc += cw[i * TAPS + j] * hist[k][j];
+    for (int j = 0; j < K; j++) acc += wt[k][j] * hist[k][j];
     out[(int64_t)t * W + i] = from_f<T>(acc);
     if (live) {
 #pragma unroll

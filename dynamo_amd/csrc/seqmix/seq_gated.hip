@@ -219,10 +219,12 @@ DEVINL void wave_argmax(float& v, int& i) {
 // are out of the running; the `top` largest remaining choices are taken in
 // falling order and weigh in with s * scale.
 // LDS per wave: s [n], choice [n], group score [groups].
-// The logits are given (fp32 [T, n]), or - for few rows - formed here as
-// the fp32 products of the token's input h [W] (activation type) with the
-// router's fp32 rows [n, W], eight outputs at a time.
-template <typename T>
+// The logits are given (fp32 [T, n]; a wave per token, four tokens per
+// workgroup), or - FUSED, for few rows - formed here as the fp32 products of
+// the token's input h [W] (activation type) with the router's fp32 rows
+// [n, W]: then a workgroup owns one token, all its threads share the
+// channels, eight outputs at a time, and its first wave routes.
+template <typename T, bool FUSED>
 __global__ __launch_bounds__(256) void moe_route_kernel(
     int* __restrict__ idx, float* __restrict__ wgt,
     const float* __restrict__ logits, const T* __restrict__ h,
@@ -231,20 +233,22 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
     int T_, int n, int groups, int keep, int top, float scale) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int t = blockIdx.x * 4 + wave;
+  const int t = FUSED ? blockIdx.x : blockIdx.x * 4 + wave;
   if (t >= T_) return;
-  float* sc = lds + wave * (2 * n + groups);
+  float* sc = lds + (FUSED ? 0 : wave) * (2 * n + groups);
   float* ch = sc + n;
   float* gs = ch + n;
-  if (logits) {
+  if (!FUSED) {
     for (int i = lane; i < n; i += 64) ch[i] = logits[(int64_t)t * n + i];
   } else {
+    __shared__ float part[4][8];
     const T* hr = h + (int64_t)t * W;
     for (int i0 = 0; i0 < n; i0 += 8) {
       float acc[8];
 #pragma unroll
       for (int u = 0; u < 8; u++) acc[u] = 0.f;
-      for (int c = lane; c < W; c += 64) {
+#pragma unroll 2
+      for (int c = threadIdx.x; c < W; c += 256) {
         const float hv = to_f(hr[c]);
 #pragma unroll
         for (int u = 0; u < 8; u++)
@@ -253,9 +257,15 @@ __global__ __launch_bounds__(256) void moe_route_kernel(
 #pragma unroll
       for (int u = 0; u < 8; u++) {
         const float v = wave_sum(acc[u]);
-        if (lane == 0 && i0 + u < n) ch[i0 + u] = v;
+        if (lane == 0) part[wave][u] = v;
       }
+      __syncthreads();
+      if (threadIdx.x < 8 && i0 + threadIdx.x < n)
+        ch[i0 + threadIdx.x] = (part[0][threadIdx.x] + part[1][threadIdx.x]) +
+                               (part[2][threadIdx.x] + part[3][threadIdx.x]);
+      __syncthreads();
     }
+    if (wave != 0) return;
   }
   wave_sync();
   const float* z = ch;  // raw logits, replaced by the choice scores below
@@ -380,22 +390,26 @@ __global__ void moe_combine_kernel(
     const int* __restrict__ idx, const float* __restrict__ wgt,
     const int* __restrict__ rank, const int* __restrict__ base,
     const T* __restrict__ shared, int E, int W, int top, int rows) {
+  constexpr int MAXTOP = 64;  // checked on the host
+  __shared__ const T* src[MAXTOP];
+  __shared__ float wj[MAXTOP];
   const int t = blockIdx.x;
   const T* hr = h + (int64_t)t * W;
+  // the rows this token sums, looked up once
+  for (int j = threadIdx.x; j < top; j += blockDim.x) {
+    const int e = idx[(int64_t)t * top + j];
+    wj[j] = wgt[(int64_t)t * top + j];
+    if (e >= E || e < 0) {
+      src[j] = hr;
+    } else {
+      const int r = min(max(base[e] + rank[(int64_t)t * top + j], 0), rows - 1);
+      src[j] = y + (int64_t)r * W;
+    }
+  }
+  __syncthreads();
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float acc = 0.f;
-    for (int j = 0; j < top; j++) {
-      const int e = idx[(int64_t)t * top + j];
-      const float w = wgt[(int64_t)t * top + j];
-      float v;
-      if (e >= E || e < 0) {
-        v = to_f(hr[c]);
-      } else {
-        const int r = min(max(base[e] + rank[(int64_t)t * top + j], 0), rows - 1);
-        v = to_f(y[(int64_t)r * W + c]);
-      }
-      acc += w * v;
-    }
+    for (int j = 0; j < top; j++) acc += wj[j] * to_f(src[j][c]);
     if (shared) acc += to_f(shared[(int64_t)t * W + c]);
     out[(int64_t)t * W + c] = from_f<T>(acc);
   }
@@ -556,14 +570,15 @@ void moe_route(torch::Tensor idx, torch::Tensor wgt, torch::Tensor logits,
   if (T_ == 0) return;
   if (router) {
     DISPATCH_ACT(logits, hipLaunchKernelGGL(
-        moe_route_kernel<T>, dim3((T_ + 3) / 4), dim3(256), lds, cur_stream(),
+        (moe_route_kernel<T, true>), dim3(T_), dim3(256), lds, cur_stream(),
         ptr<int>(idx), ptr<float>(wgt), (const float*)nullptr,
         cptr<T>(logits), cptr<float>(*router), (int)logits.size(1),
         cptr<float>(correction), T_, n, (int)groups, (int)keep, top,
         (float)scale););
   } else {
-    hipLaunchKernelGGL(moe_route_kernel<float>, dim3((T_ + 3) / 4), dim3(256),
-                       lds, cur_stream(), ptr<int>(idx), ptr<float>(wgt),
+    hipLaunchKernelGGL((moe_route_kernel<float, false>), dim3((T_ + 3) / 4),
+                       dim3(256), lds, cur_stream(), ptr<int>(idx),
+                       ptr<float>(wgt),
                        cptr<float>(logits), (const float*)nullptr,
                        (const float*)nullptr, 0, cptr<float>(correction), T_,
                        n, (int)groups, (int)keep, top, (float)scale);
@@ -621,6 +636,7 @@ void moe_combine(torch::Tensor out, torch::Tensor y, torch::Tensor h,
                 wgt.scalar_type() == torch::kFloat && wgt.is_contiguous() &&
                 wgt.numel() == idx.numel(), "combine choices");
   check_ints(base, E, "base");
+  SEQ_CHECK(top >= 1 && top <= 64, "experts per token");
   if (shared)
     SEQ_CHECK(shared->is_contiguous() && shared->dim() == 2 &&
                   shared->size(0) == T_ && shared->size(1) == W &&
