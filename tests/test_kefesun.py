@@ -715,3 +715,64 @@ def test_graph_decode_matches_eager(full_ckpt):
         for so in eng.step():
             out[so.req_id].append(so.new_token)
     assert out == want
+
+
+def test_preset_and_state_declaration():
+    """The random-weight preset builds, declares its caches and state, and
+    generates through the scheduler; identity and grouped routers, a layer
+    without feed-forward and one without window are all in it."""
+    from dynamo_amd.engine import EngineConfig, LLMEngine, SamplingParams
+    from dynamo_amd.engine.config import PRESETS
+    from dynamo_amd.models.registry import native_extensions
+    cfg = PRESETS["tiny-kefesun"]
+    assert native_extensions(cfg, "cuda:0") == ["_core", "_hip_seq"]
+    eng = LLMEngine(EngineConfig(model=cfg, device="cpu", dtype="float32",
+                                 page_size=16, max_num_seqs=2,
+                                 max_model_len=128, kv_pool_pages=12,
+                                 enable_hip_graphs=False), seed=0)
+    model = eng.runner.model
+    K, W = cfg.conv_taps - 1, cfg.hidden_size
+    assert model.kv_layer_shapes() == [(2, 24, 16), None, (1, 16, 24)]
+    assert model.state_layer_shapes() == [[(K, W), (K, W)], [(K, W), (72,)],
+                                          [(K, W), (K, W)]]
+    eng.add_request("a", list(range(3, 40)),
+                    SamplingParams(max_tokens=4, temperature=0.0,
+                                   ignore_eos=True))
+    out = []
+    for _ in range(50):
+        if not eng.has_work():
+            break
+        out += [so.new_token for so in eng.step()]
+    assert len(out) == 4 and eng.state_slots.num_free == 2
+
+
+def test_trace_run_command(full_ckpt, tmp_path):
+    """The command-line replay: two requests sharing steps, portions beside
+    single tokens, logits written only where they are wanted."""
+    import subprocess
+    import numpy as np
+    path, cfg, W = full_ckpt
+    a, b = U.tokens_for(cfg, 20, 40), U.tokens_for(cfg, 9, 41)
+    E = lambda i, t, w: {"id": i, "tokens": t, "want": w}  # noqa: E731
+    steps = [{"step": 0, "entries": [E("a", a[:13], [0, 12]), E("b", b[:2], [])],
+              "end": []},
+             {"step": 1, "entries": [E("a", a[13:14], []), E("b", b[2:3], [])],
+              "end": []},
+             {"step": 2, "entries": [E("b", b[3:], [5]), E("a", a[14:], [5])],
+              "end": ["a", "b"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", path,
+                        "--dtype", "float32", "--out", str(tmp_path / "o"),
+                        "--max-tokens", "128", "--device", "cpu"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n",
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [x for x in r.stdout.splitlines() if x.startswith("done")] == \
+        ["done 0", "done 1", "done 2"]
+    wa, wb = oracle.forward(cfg, W, a), oracle.forward(cfg, W, b)
+    first = np.fromfile(tmp_path / "o" / "0.f32", dtype="<f4").reshape(2, -1)
+    last = np.fromfile(tmp_path / "o" / "2.f32", dtype="<f4").reshape(2, -1)
+    assert not (tmp_path / "o" / "1.f32").exists()
+    got = torch.from_numpy(np.concatenate([first, last]))
+    want = torch.stack([wa[0], wa[12], wb[8], wa[19]])
+    assert U.rel_err(got, want) < U.TOL["float32"]
