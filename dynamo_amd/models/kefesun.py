@@ -146,6 +146,10 @@ class KefesunForCausalLM(torch.nn.Module):
                 _put(layer.norm2, get(p + "norm2"))
                 layer.mlp.load(lambda n, p=p: get(p + "mlp." + n))
         extra = set(tensors) - used
+        # a layer without feed-forward has no use for a second norm or
+        # convolution, should a checkpoint carry them
+        extra -= {f"l{i}.{n}" for i, layer in enumerate(self.layers)
+                  if layer.mlp is None for n in ("norm2", "canon2")}
         if extra:
             raise ValueError(f"checkpoint tensors not consumed: {sorted(extra)}")
         return len(used)
