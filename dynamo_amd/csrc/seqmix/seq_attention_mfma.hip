@@ -17,8 +17,12 @@
 // 16-byte run of keys. Large rows (a 576-wide latent row with 512 value
 // channels) therefore need no more LDS than small ones. The fp32 scores
 // get the row's temperature and scale, the distance penalty and the mask,
-// then an online softmax; the weights pass through LDS as a bf16 hi + lo
-// pair to become the A operand of two products.
+// then an online softmax. Both products are formed transposed
+// (S^T = K Q^T, O^T = V^T P^T): a lane then holds the scores of one query
+// row, and the weights it computes are, as they lie in its registers, the
+// B operand of the second product - as a bf16 hi + lo pair, i.e. two
+// products - without passing through LDS. The keys of a block are staged
+// for the second product in the order in which the lanes hold them.
 //
 // Decoded tokens use the same kernel with the roles of the tile's rows
 // changed (HEADS): a tile is one token, its rows are the query heads that
@@ -31,6 +35,13 @@
 // lg = l / 16):  A: A[row = lr][k = 8 lg + i], i = 0..7
 //                B: B[k = 8 lg + i][col = lr]
 //                D: D[row = 4 lg + r][col = lr], r = 0..3
+// S^T block n: A = keys 16 n + (0..15) (rows) x channels, B = Q^T, so
+// lane (lr, lg) gets the scores of query row lr with keys 16 n + 4 lg + r.
+// O^T: A = V^T (16 channels x 32 keys), B = P^T: lane (lr, lg) supplies
+// the weights of query row lr for 8 keys of the 32 - those it holds: of
+// half kt of the block, key 32 kt + 16 a + 4 lg + r sits at position
+// 32 kt + 8 lg + 4 a + r of the staged value rows. D = O^T[channel 4 lg + r
+// of the 16][query row lr].
 #include "seq_common.h"
 
 namespace {
@@ -71,12 +82,10 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   constexpr int DCH = DN < 8 ? DN : 8;       // value chunk: DCH * 16 channels
   constexpr int NDCH = (DN + DCH - 1) / DCH;
   constexpr int KS = KCH * 32 + PADE;  // k_lds row stride (elements)
-  constexpr int VS = BN + PADE;        // vt_lds / p_lds row stride
-  static_assert(BN * KS >= 4 * 16 * VS, "the K block also holds the lo weights");
+  constexpr int VS = BN + PADE;        // vt_lds row stride
   extern __shared__ __attribute__((aligned(16))) short smem[];
   short* k_lds = smem;                    // [BN][KS]
   short* vt_lds = k_lds + BN * KS;        // [DCH * 16][VS]
-  short* p_lds = vt_lds + DCH * 16 * VS;  // [4][16][VS]
 
   const int H = a.H, G = a.G, dk = a.dk, dv = a.dv, ps = a.ps;
   const int tile = blockIdx.x;
@@ -120,29 +129,21 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       q_frag[kc] = *reinterpret_cast<bf16x8_t*>(&v);
     }
   }
-  // ---- the 4 score rows this lane holds: wid*16 + 4 lg + r
-  int pos_r[4];
-  float qmul[4];
-  bool ok_r[4];
-#pragma unroll
-  for (int r = 0; r < 4; r++) {
-    const int cr = wid * 16 + lg * 4 + r;
-    ok_r[r] = cr < nrows;
-    pos_r[r] = HEADS ? a.positions[row0]
-                     : (ok_r[r] ? a.positions[row0 + cr] : 0);
-    float temp = 1.f;
-    if (a.temp_coef != 0.f)
-      temp += a.temp_coef * logf((float)((pos_r[r] + 1) / a.temp_every) + 1.f);
-    qmul[r] = temp * a.scale;
-  }
+  // ---- the query row whose scores this lane holds: wid*16 + lr
+  const int my_row = wid * 16 + lr;
+  const bool my_ok = my_row < nrows;
+  const int my_pos = HEADS ? a.positions[row0]
+                           : (my_ok ? a.positions[row0 + my_row] : 0);
+  float my_qmul = a.scale;
+  if (a.temp_coef != 0.f)
+    my_qmul *= 1.f + a.temp_coef *
+                         logf((float)((my_pos + 1) / a.temp_every) + 1.f);
   const float b1 = a.has_bias ? a.r1[h] : 0.f;
   const float b2 = a.has_bias ? a.r2[h] : 0.f;
-  float hb[4];  // constant added to the scaled scores of each row's head
-#pragma unroll
-  for (int r = 0; r < 4; r++)
-    hb[r] = !a.head_bias ? 0.f
-            : HEADS ? (ok_r[r] ? a.head_bias[h + wid * 16 + lg * 4 + r] : 0.f)
-                    : a.head_bias[h];
+  // constant added to the scaled scores of the row's head
+  const float my_hb = !a.head_bias ? 0.f
+                      : HEADS ? (my_ok ? a.head_bias[h + my_row] : 0.f)
+                              : a.head_bias[h];
   // prompt rows are in order; the heads of a token share its position
   const int kv_end = a.positions[HEADS ? row0 : row0 + nrows - 1] + 1;
   // the first key any row of the tile sees
@@ -150,13 +151,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int kv_begin =
       window > 0 ? max(0, a.positions[row0] - window + 1) : 0;
 
-  float m[4], l[4];
-  f32x4_t acc_o[DN];
-#pragma unroll
-  for (int r = 0; r < 4; r++) {
-    m[r] = -INFINITY;
-    l[r] = 0.f;
-  }
+  float m = -INFINITY, l = 0.f;
+  f32x4_t acc_o[DN];  // O^T: channels 16 d + 4 lg + r of query row lr
 #pragma unroll
   for (int d = 0; d < DN; d++) acc_o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
@@ -215,8 +211,11 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       const int v = slot / BN, row = slot - v * BN;
       const bool ok = t0 + row < kv_end && (vc * DCH * 2 + v) * 8 < dv;
       const short8_t x = ok ? stage[u] : short8_t{};
+      // key 32 kt + 16 a + 4 g + r of the block goes to 32 kt + 8 g + 4 a + r
+      const int col = (row & 32) | ((row & 12) << 1) | ((row & 16) >> 2) |
+                      (row & 3);
 #pragma unroll
-      for (int e = 0; e < 8; e++) vt_lds[(v * 8 + e) * VS + row] = x[e];
+      for (int e = 0; e < 8; e++) vt_lds[(v * 8 + e) * VS + col] = x[e];
     }
   };
 
@@ -235,8 +234,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   if (vb_first < nvb) load_k(block_t0(vb_first), 0);
   for (int vb = vb_first; vb < nvb; vb += vstep) {
     const int t0 = block_t0(vb);
-    // ---- S = Q K^T over key-channel chunks: block n covers keys
-    //      t0 + 16 n + lr
+    // ---- S^T = K Q^T over key-channel chunks: s[n][r] is the score of
+    //      query row lr with key t0 + 16 n + 4 lg + r
     f32x4_t s[4];
 #pragma unroll
     for (int n = 0; n < 4; n++) s[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -256,83 +255,86 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
             short8_t kb = *reinterpret_cast<const short8_t*>(
                 k_lds + (n * 16 + lr) * KS + kc * 32 + lg * 8);
             s[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                q_frag[cc * KCH + kc], *reinterpret_cast<bf16x8_t*>(&kb), s[n],
+                *reinterpret_cast<bf16x8_t*>(&kb), q_frag[cc * KCH + kc], s[n],
                 0, 0, 0);
           }
         }
       }
     }
-    // ---- fp32: scale, penalty, mask, online softmax (rows 4 lg + r)
+    // ---- fp32: scale, penalty, mask, weights of query row lr
     float p[4][4];
     if (a.sigmoid) {
       // unnormalised weights: no running maximum, no rescaling
 #pragma unroll
-      for (int r = 0; r < 4; r++)
+      for (int n = 0; n < 4; n++)
 #pragma unroll
-        for (int n = 0; n < 4; n++) {
-          const int j = t0 + n * 16 + lr;
-          const bool seen =
-              j <= pos_r[r] && (window == 0 || j > pos_r[r] - window ||
-                                j < a.keep_first);
-          p[n][r] = seen ? sigmoid_f(s[n][r] * qmul[r] + hb[r]) : 0.f;
+        for (int r = 0; r < 4; r++) {
+          const int j = t0 + n * 16 + lg * 4 + r;
+          const bool seen = j <= my_pos && (window == 0 || j > my_pos - window ||
+                                            j < a.keep_first);
+          p[n][r] = seen ? sigmoid_f(s[n][r] * my_qmul + my_hb) : 0.f;
         }
-    } else
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
+    } else {
       float mt = -INFINITY;
 #pragma unroll
-      for (int n = 0; n < 4; n++) {
-        const int j = t0 + n * 16 + lr;
-        float x = s[n][r] * qmul[r] + hb[r];
-        if (a.has_bias) x -= b1 * log1pf(b2 * (float)max(pos_r[r] - j, 0));
-        const bool seen =
-            j <= pos_r[r] && (window == 0 || j > pos_r[r] - window ||
-                              j < a.keep_first);
-        x = seen ? x : -INFINITY;
-        p[n][r] = x;
-        mt = fmaxf(mt, x);
-      }
-      mt = fmaxf(mt, __shfl_xor(mt, 1, 64));
-      mt = fmaxf(mt, __shfl_xor(mt, 2, 64));
-      mt = fmaxf(mt, __shfl_xor(mt, 4, 64));
-      mt = fmaxf(mt, __shfl_xor(mt, 8, 64));
+      for (int n = 0; n < 4; n++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+          const int j = t0 + n * 16 + lg * 4 + r;
+          float x = s[n][r] * my_qmul + my_hb;
+          if (a.has_bias) x -= b1 * log1pf(b2 * (float)max(my_pos - j, 0));
+          const bool seen = j <= my_pos && (window == 0 || j > my_pos - window ||
+                                            j < a.keep_first);
+          x = seen ? x : -INFINITY;
+          p[n][r] = x;
+          mt = fmaxf(mt, x);
+        }
+      // the row's keys are spread over the four lane groups
+      mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
       // a row may see nothing of the first blocks (window): then every
       // weight is 0 and the running maximum stays -inf
-      const float mn = fmaxf(m[r], mt);
+      const float mn = fmaxf(m, mt);
       const float base = mn == -INFINITY ? 0.f : mn;
-      const float corr = expf(m[r] - base);
+      const float corr = expf(m - base);
       float rs = 0.f;
 #pragma unroll
-      for (int n = 0; n < 4; n++) {
-        p[n][r] = expf(p[n][r] - base);
-        rs += p[n][r];
-      }
-      rs += __shfl_xor(rs, 1, 64);
-      rs += __shfl_xor(rs, 2, 64);
-      rs += __shfl_xor(rs, 4, 64);
-      rs += __shfl_xor(rs, 8, 64);
-      l[r] = l[r] * corr + rs;
-      m[r] = mn;
+      for (int n = 0; n < 4; n++)
 #pragma unroll
-      for (int d = 0; d < DN; d++) acc_o[d][r] *= corr;
+        for (int r = 0; r < 4; r++) {
+          p[n][r] = expf(p[n][r] - base);
+          rs += p[n][r];
+        }
+      rs += __shfl_xor(rs, 16, 64);
+      rs += __shfl_xor(rs, 32, 64);
+      l = l * corr + rs;
+      m = mn;
+#pragma unroll
+      for (int d = 0; d < DN; d++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc_o[d][r] *= corr;
     }
-    // ---- weights to LDS in the A layout of the second product, as a
-    // bf16 pair hi + lo (about 16 bits of mantissa, so the product below
-    // sees the fp32 weights almost exactly). lo reuses the K block, which
-    // every wave has finished reading once the barrier is passed.
-    __syncthreads();
-    short* pw = p_lds + wid * 16 * VS;
-    short* pl = k_lds + wid * 16 * VS;
+    // ---- the weights as B operands of the second product, a bf16 pair
+    // hi + lo each (about 16 bits of mantissa, so the product below sees
+    // the fp32 weights almost exactly): half kt of the block takes
+    // p[2 kt + a][r] at k index 8 lg + 4 a + r
+    bf16x8_t p_hi[2], p_lo[2];
 #pragma unroll
-    for (int r = 0; r < 4; r++)
+    for (int kt = 0; kt < 2; kt++) {
+      short8_t vh, vl;
 #pragma unroll
-      for (int n = 0; n < 4; n++) {
-        const bf16_t hi = from_f<bf16_t>(p[n][r]);
-        const bf16_t lo = from_f<bf16_t>(p[n][r] - to_f(hi));
-        pw[(lg * 4 + r) * VS + n * 16 + lr] = (short)hi;
-        pl[(lg * 4 + r) * VS + n * 16 + lr] = (short)lo;
+      for (int i = 0; i < 8; i++) {
+        const float w = p[2 * kt + (i >> 2)][i & 3];
+        const bf16_t hi = from_f<bf16_t>(w);
+        vh[i] = (short)hi;
+        vl[i] = (short)from_f<bf16_t>(w - to_f(hi));
       }
-    // ---- O += P V over value-channel chunks, V staged transposed
+      p_hi[kt] = *reinterpret_cast<bf16x8_t*>(&vh);
+      p_lo[kt] = *reinterpret_cast<bf16x8_t*>(&vl);
+    }
+    // ---- O^T += V^T P^T over value-channel chunks, V staged transposed.
+    // Every wave has passed this block's barriers after its reads of the
+    // previous block's values, so the first chunk may be written at once.
 #pragma unroll
     for (int vc = 0; vc < NDCH; vc++) {
       if (vc) __syncthreads();  // the previous chunk's readers are done
@@ -343,61 +345,52 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       if (active)
 #pragma unroll
       for (int kt = 0; kt < 2; kt++) {
-        short8_t pa = *reinterpret_cast<const short8_t*>(
-            pw + lr * VS + kt * 32 + lg * 8);
-        short8_t pb = *reinterpret_cast<const short8_t*>(
-            pl + lr * VS + kt * 32 + lg * 8);
 #pragma unroll
         for (int d = 0; d < DCH; d++) {
           if (vc * DCH + d < DN) {
             short8_t vb = *reinterpret_cast<const short8_t*>(
                 vt_lds + (d * 16 + lr) * VS + kt * 32 + lg * 8);
             acc_o[vc * DCH + d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                *reinterpret_cast<bf16x8_t*>(&pa),
-                *reinterpret_cast<bf16x8_t*>(&vb), acc_o[vc * DCH + d], 0, 0, 0);
+                *reinterpret_cast<bf16x8_t*>(&vb), p_hi[kt],
+                acc_o[vc * DCH + d], 0, 0, 0);
             acc_o[vc * DCH + d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                *reinterpret_cast<bf16x8_t*>(&pb),
-                *reinterpret_cast<bf16x8_t*>(&vb), acc_o[vc * DCH + d], 0, 0, 0);
+                *reinterpret_cast<bf16x8_t*>(&vb), p_lo[kt],
+                acc_o[vc * DCH + d], 0, 0, 0);
           }
         }
       }
     }
   }
+  if (!my_ok) return;
   if (HEADS) {
     // ---- partial result of this key split: [token, head, map, split] x
-    //      (max, sum, dv unnormalised channels)
+    //      (max, sum, dv unnormalised channels); the row is head h + my_row
+    float* o = a.partial +
+               ((((int64_t)row0 * H + h + my_row) * a.kmaps + map) * a.nsplit +
+                blockIdx.z) * (dv + 2);
+    if (lg == 0) {
+      o[0] = m;
+      o[1] = l;
+    }
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-      if (!ok_r[r]) continue;
-      const int hh = h + wid * 16 + lg * 4 + r;
-      float* o = a.partial +
-                 ((((int64_t)row0 * H + hh) * a.kmaps + map) * a.nsplit +
-                  blockIdx.z) * (dv + 2);
-      if (lr == 0) {
-        o[0] = m[r];
-        o[1] = l[r];
-      }
+    for (int d = 0; d < DN; d++)
 #pragma unroll
-      for (int d = 0; d < DN; d++) {
-        const int ch = d * 16 + lr;
+      for (int r = 0; r < 4; r++) {
+        const int ch = d * 16 + lg * 4 + r;
         if (ch < dv) o[2 + ch] = acc_o[d][r];
       }
-    }
     return;
   }
-  // ---- normalise and store rows 4 lg + r, channels 16 d + lr
+  // ---- normalise and store query row lr, channels 16 d + 4 lg + r
+  const float inv = a.sigmoid ? 1.f : 1.f / l;
+  TO* o = out + (((int64_t)(row0 + my_row) * H + h) * a.kmaps + map) * dv;
 #pragma unroll
-  for (int r = 0; r < 4; r++) {
-    if (!ok_r[r]) continue;
-    const float inv = a.sigmoid ? 1.f : 1.f / l[r];
-    TO* o = out + (((int64_t)(row0 + wid * 16 + lg * 4 + r) * H + h) * a.kmaps +
-                   map) * dv;
+  for (int d = 0; d < DN; d++)
 #pragma unroll
-    for (int d = 0; d < DN; d++) {
-      const int ch = d * 16 + lr;
+    for (int r = 0; r < 4; r++) {
+      const int ch = d * 16 + lg * 4 + r;
       if (ch < dv) o[ch] = out_cast<TO>(acc_o[d][r] * inv);
     }
-  }
 }
 
 // out[t, h, map, :] from the nsplit (<= 16) partial results of a decoded
@@ -439,8 +432,8 @@ __global__ void merge_splits_kernel(float* __restrict__ out,
 
 inline size_t lds_bytes(int KC, int DN) {
   const int KCH = KC < 4 ? KC : 4, DCH = DN < 8 ? DN : 8;
-  return (size_t)(BN * (KCH * 32 + PADE) + DCH * 16 * (BN + PADE) +
-                  4 * 16 * (BN + PADE)) * sizeof(short);
+  return (size_t)(BN * (KCH * 32 + PADE) + DCH * 16 * (BN + PADE)) *
+         sizeof(short);
 }
 
 template <int KC, int DN, typename TO>
