@@ -49,6 +49,13 @@ namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) short short8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(8))) float f32x8_t;
+
+// sigmoid from the hardware exponential and reciprocal (about 1 ulp each;
+// the weights are used with 16 bits of mantissa)
+DEVINL float sigmoid_fast(float x) {
+  return __builtin_amdgcn_rcpf(1.f + __expf(-x));
+}
 
 constexpr int BN = 64;    // keys per block
 constexpr int PADE = 8;   // padding elements per LDS row (16 bytes)
@@ -88,16 +95,30 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   short* vt_lds = k_lds + BN * KS;        // [DCH * 16][VS]
 
   const int H = a.H, G = a.G, dk = a.dk, dv = a.dv, ps = a.ps;
-  const int tile = blockIdx.x;
+  // Workgroups go to the 8 XCDs in turn by their linear index, each XCD
+  // with an L2 of its own. Prompt tiles are renumbered so that an XCD gets
+  // a contiguous run of (head, tile) pairs: the tiles of a head - and of
+  // the heads that share its keys and values - then meet in one L2 instead
+  // of every XCD streaming every sequence's keys.
+  int bx = blockIdx.x, by = blockIdx.y;
+  if (!HEADS) {
+    const int total = gridDim.x * gridDim.y;
+    if (total % 8 == 0) {
+      const int lin = bx + gridDim.x * by;
+      const int w = (lin % 8) * (total / 8) + lin / 8;
+      bx = w % gridDim.x;
+      by = w / gridDim.x;
+    }
+  }
+  const int tile = bx;
   const int gsz = H / G;
   // prompt tiles: blockIdx.y = head * kmaps + map, rows are tokens.
   // HEADS: blockIdx.y = ((kv head * kmaps) + map) * nhb + head block,
   // blockIdx.x is the token and rows are the heads h0 + row.
   const int nhb = (gsz + 63) / 64;
-  const int map = HEADS ? (blockIdx.y / nhb) % a.kmaps : blockIdx.y % a.kmaps;
-  const int g = HEADS ? blockIdx.y / (nhb * a.kmaps)
-                      : (blockIdx.y / a.kmaps) / gsz;
-  const int h = HEADS ? g * gsz + (blockIdx.y % nhb) * 64 : blockIdx.y / a.kmaps;
+  const int map = HEADS ? (by / nhb) % a.kmaps : by % a.kmaps;
+  const int g = HEADS ? by / (nhb * a.kmaps) : (by / a.kmaps) / gsz;
+  const int h = HEADS ? g * gsz + (by % nhb) * 64 : by / a.kmaps;
   const int koff = map * dk;
   const int row0 = HEADS ? tile : a.tile_row0[tile];
   const int nrows = HEADS ? min(64, g * gsz + gsz - h) : a.tile_rows[tile];
@@ -166,6 +187,21 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   // Loads are unconditional with clamped addresses (a branch around a load
   // would make each wait for the one before); what lies past the end of
   // the keys or of the row is zeroed when the piece is written to LDS.
+  // slot of key j: page index and place in the page (shift and mask when
+  // the page size is a power of two)
+  const bool ps_pow2 = (ps & (ps - 1)) == 0;
+  const int ps_shift = __ffs(ps) - 1;
+  auto key_row = [&](int j) -> int64_t {
+    int pg, in;
+    if (ps_pow2) {
+      pg = j >> ps_shift;
+      in = j & (ps - 1);
+    } else {
+      pg = j / ps;
+      in = j - pg * ps;
+    }
+    return ((int64_t)table[pg] * G + g) * ps + in;
+  };
   auto load_k = [&](int t0, int cc) {
     constexpr int kvecs = KCH * 4;  // 16-byte pieces per staged row
 #pragma unroll
@@ -174,9 +210,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       const int row = slot / kvecs, v = slot - row * kvecs;
       const int j = min(t0 + row, kv_end - 1);
       const int ch = min((cc * KCH * 4 + v) * 8, dk - 8);
-      const int64_t page = table[j / ps];
       stage[u] = *reinterpret_cast<const short8_t*>(
-          a.kcache + ((page * G + g) * ps + (j % ps)) * a.krow + koff + ch);
+          a.kcache + key_row(j) * a.krow + koff + ch);
     }
   };
   auto store_k = [&](int t0, int cc) {
@@ -199,9 +234,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
       const int v = slot / BN, row = slot - v * BN;
       const int j = min(t0 + row, kv_end - 1);
       const int ch = min((vc * DCH * 2 + v) * 8, dv - 8);
-      const int64_t page = table[j / ps];
       stage[u] = *reinterpret_cast<const short8_t*>(
-          a.vcache + ((page * G + g) * ps + (j % ps)) * a.vrow + ch);
+          a.vcache + key_row(j) * a.vrow + ch);
     }
   };
   auto store_v = [&](int t0, int vc) {
@@ -272,7 +306,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
           const int j = t0 + n * 16 + lg * 4 + r;
           const bool seen = j <= my_pos && (window == 0 || j > my_pos - window ||
                                             j < a.keep_first);
-          p[n][r] = seen ? sigmoid_f(s[n][r] * my_qmul + my_hb) : 0.f;
+          p[n][r] = seen ? sigmoid_fast(s[n][r] * my_qmul + my_hb) : 0.f;
         }
     } else {
       float mt = -INFINITY;
@@ -321,16 +355,13 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     bf16x8_t p_hi[2], p_lo[2];
 #pragma unroll
     for (int kt = 0; kt < 2; kt++) {
-      short8_t vh, vl;
+      f32x8_t w;
 #pragma unroll
-      for (int i = 0; i < 8; i++) {
-        const float w = p[2 * kt + (i >> 2)][i & 3];
-        const bf16_t hi = from_f<bf16_t>(w);
-        vh[i] = (short)hi;
-        vl[i] = (short)from_f<bf16_t>(w - to_f(hi));
-      }
-      p_hi[kt] = *reinterpret_cast<bf16x8_t*>(&vh);
-      p_lo[kt] = *reinterpret_cast<bf16x8_t*>(&vl);
+      for (int i = 0; i < 8; i++) w[i] = p[2 * kt + (i >> 2)][i & 3];
+      // vector conversions (round to nearest even): packed converts
+      p_hi[kt] = __builtin_convertvector(w, bf16x8_t);
+      p_lo[kt] = __builtin_convertvector(
+          w - __builtin_convertvector(p_hi[kt], f32x8_t), bf16x8_t);
     }
     // ---- O^T += V^T P^T over value-channel chunks, V staged transposed.
     // Every wave has passed this block's barriers after its reads of the
