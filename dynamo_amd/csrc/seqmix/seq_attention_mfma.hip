@@ -169,8 +169,8 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const int kv_end = a.positions[HEADS ? row0 : row0 + nrows - 1] + 1;
   // the first key any row of the tile sees
   const int window = a.window;
-  const int kv_begin =
-      window > 0 ? max(0, a.positions[row0] - window + 1) : 0;
+  const int pos_first = a.positions[row0];  // smallest position of the tile
+  const int kv_begin = window > 0 ? max(0, pos_first - window + 1) : 0;
 
   float m = -INFINITY, l = 0.f;
   f32x4_t acc_o[DN];  // O^T: channels 16 d + 4 lg + r of query row lr
@@ -202,16 +202,30 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     }
     return ((int64_t)table[pg] * G + g) * ps + in;
   };
+  // A whole block inside one page and inside the keys (all but a
+  // sequence's last block when pages are at least a block long): one page
+  // lookup for the workgroup, the rest of a thread's address never changes.
+  const bool one_page = ps_pow2 && ps >= BN;
   auto load_k = [&](int t0, int cc) {
     constexpr int kvecs = KCH * 4;  // 16-byte pieces per staged row
+    const bool fast = one_page && t0 + BN <= kv_end;
+    const bf16_t* base =
+        a.kcache +
+        ((((int64_t)table[fast ? t0 >> ps_shift : 0] * G + g) * ps +
+          (t0 & (ps - 1))) * a.krow + koff);
 #pragma unroll
     for (int u = 0; u < NSK; u++) {
       const int slot = threadIdx.x + u * 256;
       const int row = slot / kvecs, v = slot - row * kvecs;
-      const int j = min(t0 + row, kv_end - 1);
       const int ch = min((cc * KCH * 4 + v) * 8, dk - 8);
-      stage[u] = *reinterpret_cast<const short8_t*>(
-          a.kcache + key_row(j) * a.krow + koff + ch);
+      if (fast) {
+        stage[u] =
+            *reinterpret_cast<const short8_t*>(base + (row * a.krow + ch));
+      } else {
+        const int j = min(t0 + row, kv_end - 1);
+        stage[u] = *reinterpret_cast<const short8_t*>(
+            a.kcache + key_row(j) * a.krow + koff + ch);
+      }
     }
   };
   auto store_k = [&](int t0, int cc) {
@@ -228,14 +242,24 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   // consecutive threads take consecutive keys of one channel group, so the
   // transposed 2-byte LDS writes fall in consecutive banks
   auto load_v = [&](int t0, int vc) {
+    const bool fast = one_page && t0 + BN <= kv_end;
+    const bf16_t* base =
+        a.vcache +
+        (((int64_t)table[fast ? t0 >> ps_shift : 0] * G + g) * ps +
+         (t0 & (ps - 1))) * a.vrow;
 #pragma unroll
     for (int u = 0; u < NSV; u++) {
       const int slot = threadIdx.x + u * 256;
       const int v = slot / BN, row = slot - v * BN;
-      const int j = min(t0 + row, kv_end - 1);
       const int ch = min((vc * DCH * 2 + v) * 8, dv - 8);
-      stage[u] = *reinterpret_cast<const short8_t*>(
-          a.vcache + key_row(j) * a.vrow + ch);
+      if (fast) {
+        stage[u] =
+            *reinterpret_cast<const short8_t*>(base + (row * a.vrow + ch));
+      } else {
+        const int j = min(t0 + row, kv_end - 1);
+        stage[u] = *reinterpret_cast<const short8_t*>(
+            a.vcache + key_row(j) * a.vrow + ch);
+      }
     }
   };
   auto store_v = [&](int t0, int vc) {
@@ -297,7 +321,16 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     }
     // ---- fp32: scale, penalty, mask, weights of query row lr
     float p[4][4];
-    if (a.sigmoid) {
+    // every row of the tile sees every key of the block (uniform)
+    const bool all_seen =
+        t0 + BN - 1 <= pos_first && (window == 0 || t0 > kv_end - 1 - window);
+    if (a.sigmoid && all_seen) {
+#pragma unroll
+      for (int n = 0; n < 4; n++)
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          p[n][r] = sigmoid_fast(s[n][r] * my_qmul + my_hb);
+    } else if (a.sigmoid) {
       // unnormalised weights: no running maximum, no rescaling
 #pragma unroll
       for (int n = 0; n < 4; n++)
