@@ -97,14 +97,15 @@ def kefesun_config(width, layers, ff):
     """Layer pattern: three sigmoid-attention layers (128-wide heads, four
     query heads per kv head, a 1024-token window that keeps the first four
     tokens) to one minimal gated recurrent unit of the model's width; every
-    layer with eight routed experts and two identity experts in two groups,
-    two per token, and a shared expert. A token's active feed-forward
+    layer with eight routed experts and four identity experts in three
+    groups of which two stay in the running, two per token, and a shared
+    expert. A token's active feed-forward
     weights equal those of a dense gated feed-forward of size ff."""
     from dynamo_amd.engine.config import ModelConfig
     H = width // 128
     mlp = {"kind": "moe", "expert": {"ff": ff // 2},
-           "router": {"experts": 8, "identity": 2, "top": 2, "scale": 1.0,
-                      "groups": {"count": 2, "keep": 1}},
+           "router": {"experts": 8, "identity": 4, "top": 2, "scale": 1.0,
+                      "groups": {"count": 3, "keep": 2}},
            "shared": {"ff": ff // 2}}
     attn = {"type": "attention", "mlp": mlp, "mixer": {
         "heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128,

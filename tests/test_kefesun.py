@@ -202,12 +202,12 @@ def test_router_against_oracle(device, n, groups, keep, top):
     h = torch.randn(T, Wd, generator=g, dtype=torch.float64)
     Wt = {"p.router": torch.randn(n, Wd, generator=g) * 0.8,
           "p.correction": torch.rand(n, generator=g) * 0.5 - 0.45}
-    r = {"experts": n, "top": top, "scale": 2.5,
+    r = {"experts": n, "top": top, "scale": 1.7,
          "groups": {"count": groups, "keep": keep}}
     want_idx, want_w = oracle.route(h, Wt, "p.", r)
     logits = (h @ Wt["p.router"].double().t()).float().to(device)
     idx, wgt = sops.moe_route(logits, Wt["p.correction"].to(device), groups,
-                              keep, top, 2.5)
+                              keep, top, 1.7)
     assert torch.equal(idx.cpu().long().sort(-1).values,
                        want_idx.sort(-1).values)
     order = idx.cpu().long().argsort(-1)
@@ -221,7 +221,7 @@ def test_router_against_oracle(device, n, groups, keep, top):
         want_idx2, want_w2 = oracle.route(hh.double(), Wt, "p.", r)
         idx2, wgt2 = sops.moe_route_rows(
             hh.to(device), Wt["p.router"].to(device),
-            Wt["p.correction"].to(device), groups, keep, top, 2.5)
+            Wt["p.correction"].to(device), groups, keep, top, 1.7)
         same = (idx2.cpu().long().sort(-1).values
                 == want_idx2.sort(-1).values).all(-1)
         assert float(same.float().mean()) > 0.9      # near-ties may flip
@@ -416,7 +416,7 @@ def _op_attention(device, q, k, v, ps, rows, decode, window, keep, bias,
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("window,keep,ps", [(5, 2, 4), (16, 16, 16),
-                                            (64, 1, 16), (70, 6, 64),
+                                            (64, 1, 16), (70, 5, 64),
                                             (1, 3, 4), (40, 70, 16)])
 @pytest.mark.parametrize("decode", [False, True], ids=["prompt", "decoded"])
 def test_window_and_kept_edges_at_op_level(device, window, keep, ps, decode):
@@ -636,7 +636,7 @@ def test_unused_checkpoint_tensor_is_an_error(tmp_path):
 @pytest.mark.parametrize("H,G,dk,dv,window,keep", [
     (4, 2, 64, 128, 100, 3),
     (6, 3, 24, 40, 19, 70),         # sizes padded inside the kernel
-    (2, 1, 128, 48, 0, 0),          # every earlier key visible
+    (2, 1, 128, 56, 0, 0),          # every earlier key visible
     (2, 2, 16, 8, 1, 2),            # a window of one token
     (16, 1, 64, 64, 50, 1),
 ])
