@@ -660,6 +660,17 @@ def test_mfma_sigmoid_attention_matches_oracle(H, G, dk, dv, window, keep):
                 dk ** -0.5, float(bias[hh]), window or None, keep)[rows]
             err = (got[:, hh].double() - want).abs().max() / want.abs().max()
             assert float(err) < 1e-2, (hh, rows[0])
+    # the last row as a decoded token: head groups of eight and more run on
+    # the matrix cores with their keys split over workgroups, the others on
+    # the row kernel
+    got = _op_attention("cuda:0", q, k, v, 16, [T - 1], True, window, keep,
+                        bias, scale=dk ** -0.5, dtype=torch.bfloat16)
+    for hh in range(H):
+        want = _sigmoid_attention_oracle(
+            q[:, hh], k[:, hh // (H // G)], v[:, hh // (H // G)], dk ** -0.5,
+            float(bias[hh]), window or None, keep)[T - 1]
+        err = (got[0, hh].double() - want).abs().max() / want.abs().max()
+        assert float(err) < 1e-2, hh
 
 
 # -- the engine's own entry point ---------------------------------------------
