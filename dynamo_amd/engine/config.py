@@ -16,7 +16,7 @@ from typing import Optional
 @dataclass
 class ModelConfig:
     name: str = "llama-3-8b"
-    arch: str = "llama"            # llama | opt | mixtral | qwen2 | bolatar | fironex | kefesun
+    arch: str = "llama"            # llama | opt | mixtral | qwen2 | bolatar | fironex | kefesun | muzulorn
     hidden_size: int = 4096
     intermediate_size: int = 14336
     num_layers: int = 32
@@ -46,6 +46,8 @@ class ModelConfig:
     logit_softcap: float = 0.0     # cap * tanh(logits / cap); 0 = off
     residual_mult: float = 1.0     # scales a normed sublayer output (fironex)
     conv_taps: int = 0             # taps of the sublayers' input convolution (kefesun)
+    residual_streams: int = 0      # parallel residual streams with learned connections; 0 = plain residual (muzulorn)
+    pair_hash: Optional[dict] = None   # {"buckets", "mul_prev", "mul_cur"}: embedding row added by a hash of the previous and current token (muzulorn)
     # local HF checkpoint dir to load real weights from ("" = random init)
     weights_path: str = ""
 

@@ -487,28 +487,48 @@ class LatentAttention(torch.nn.Module):
     all heads are stored. Head keys W_uk c and values W_uv c are never
     materialised: W_uk is folded into the query and W_uv applied to the
     attention-weighted latent, so the kernel runs as multi-query attention
-    whose values are the first `rank` entries of the cached rows. Rotation
-    pairs (i, i + dims/2) over the rot_dim part; per-head sigmoid output
-    gate. With shared_cache the layer has no down-projection of its own and
-    reads another latent layer's cache."""
+    whose values are the first `rank` entries of the cached rows. With
+    shared_cache the layer has no down-projection of its own and reads
+    another latent layer's cache.
+
+    Options: rotation pairs (i, i + dims/2) or interleaved (2i, 2i + 1)
+    over the rot_dim part; queries projected directly or through an
+    RMS-normed latent of q_rank entries (W_uq norm(W_dq h)); a sliding
+    window; a per-head sink in the softmax denominator; the output gate
+    sigmoid(W_g h) one value per head ("head", applied before W_uv, with
+    which it commutes) or one per output channel ("element", applied to the
+    concatenated heads)."""
 
     def __init__(self, width, heads, dim, rot_dim, vdim, rank, scale, rot, eps,
-                 init, shared_cache=False):
+                 init, shared_cache=False, interleaved=False, q_rank=None,
+                 window=None, sink=False, gate="head"):
         super().__init__()
+        if gate not in ("head", "element"):
+            raise ValueError(f"unknown output gate {gate!r}")
         self.W, self.H, self.dk, self.rd, self.dv = width, heads, dim, rot_dim, vdim
         self.rank, self.scale, self.eps = rank, scale, eps
         self.shared_cache = shared_cache
+        self.interleaved, self.gate = interleaved, gate
+        self.q_rank = int(q_rank or 0)
+        self.window = int(window or 0)
         self.freqs = rotary_frequencies(rot).to(init.device)
         if 2 * self.freqs.shape[1] > rot_dim:
             raise ValueError("rotary dims exceed the rotated part")
-        self.off_z = heads * (dim + rot_dim)
+        nq = heads * (dim + rot_dim)
+        self.off_z = self.q_rank or nq
         self.off_g = self.off_z + (0 if shared_cache else rank + rot_dim)
-        # fused rows: q | [latent down-projection] | gate
-        self.w_in = init.mat(self.off_g + heads, width)
+        ng = heads if gate == "head" else heads * vdim
+        # fused rows: q (or its latent) | [latent down-projection] | gate
+        self.w_in = init.mat(self.off_g + ng, width)
+        self.dq_norm = self.w_uq = None
+        if self.q_rank:
+            self.dq_norm = init.vec(self.q_rank, 0.7, 1.3)
+            self.w_uq = init.mat(nq, self.q_rank)
         self.dkv_norm = None if shared_cache else init.vec(rank, 0.7, 1.3)
         self.w_uk = torch.stack([init.mat(dim, rank) for _ in range(heads)])
         self.w_uv_t = torch.stack([init.mat(vdim, rank).t().contiguous()
                                    for _ in range(heads)])
+        self.sink = init.vec(heads, -1.0, 1.0) if sink else None
         self.w_o = init.mat(width, heads * vdim)
 
     def state_shapes(self):
@@ -518,13 +538,19 @@ class LatentAttention(torch.nn.Module):
         return None if self.shared_cache else (1, self.rank + self.rd, 0)
 
     def load(self, get: Getter):
-        rows = [get("q")] + ([] if self.shared_cache else [get("dkv")])
+        rows = [get("dq") if self.q_rank else get("q")]
+        rows += [] if self.shared_cache else [get("dkv")]
         _put(self.w_in, torch.cat(rows + [get("g")], 0))
+        if self.q_rank:
+            _put(self.dq_norm, get("dq.norm"))
+            _put(self.w_uq, get("uq"))
         if not self.shared_cache:
             _put(self.dkv_norm, get("dkv.norm"))
         _put(self.w_uk, get("uk").view(self.H, self.dk, self.rank))
         _put(self.w_uv_t, get("uv").view(self.H, self.dv,
                                          self.rank).transpose(1, 2))
+        if self.sink is not None:
+            _put(self.sink, get("sink"))
         _put(self.w_o, get("o"))
 
     def forward(self, h, ctx: MixContext):
@@ -533,20 +559,33 @@ class LatentAttention(torch.nn.Module):
         if not self.shared_cache:
             sops.latent_append(ctx.kcache, proj, self.off_z, self.dkv_norm,
                                ctx.slot_mapping, ctx.positions, self.freqs,
-                               False, self.eps)
-        qh = proj[:, :self.off_z].view(T, H, self.dk + rd)
+                               self.interleaved, self.eps)
+        if self.q_rank:
+            cq = sops.rms_norm_cols(proj, 0, self.q_rank, self.dq_norm,
+                                    self.eps, h.dtype)
+            qsrc = F.linear(cq, self.w_uq)
+        else:
+            qsrc = proj
+        qh = qsrc[:, :H * (self.dk + rd)].view(T, H, self.dk + rd)
         q = torch.empty(T, H * (R + rd), dtype=h.dtype, device=h.device)
         q.view(T, H, R + rd)[:, :, :R].copy_(
             torch.bmm(qh[:, :, :self.dk].transpose(0, 1),
                       self.w_uk).transpose(0, 1))
-        sops.rope_rows(q, R, R + rd, proj, self.dk, self.dk + rd,
-                       ctx.positions, self.freqs, H, rd, False)
+        sops.rope_rows(q, R, R + rd, qsrc, self.dk, self.dk + rd,
+                       ctx.positions, self.freqs, H, rd, self.interleaved)
         lat = sops.paged_attention_rows(q, 0, H, 1, ctx.kcache, None, R,
-                                        ctx.positions, ctx.sb, self.scale, 0)
-        g = sops.head_sigmoid_scale(lat.view(T, H, R), proj[:, self.off_g:],
-                                    h.dtype)
-        o = torch.bmm(g, self.w_uv_t)                       # [H, T, dv]
-        return F.linear(o.transpose(0, 1).reshape(T, H * self.dv), self.w_o)
+                                        ctx.positions, ctx.sb, self.scale,
+                                        self.window, sink=self.sink)
+        if self.gate == "head":
+            g = sops.head_sigmoid_scale(lat.view(T, H, R),
+                                        proj[:, self.off_g:], h.dtype)
+            o = torch.bmm(g, self.w_uv_t)                   # [H, T, dv]
+            y = o.transpose(0, 1).reshape(T, H * self.dv)
+        else:
+            o = torch.bmm(sops.heads_major(lat.view(T, H, R), h.dtype),
+                          self.w_uv_t)
+            y = sops.heads_gate(o, proj[:, self.off_g:], h.dtype)
+        return F.linear(y, self.w_o)
 
 
 class XIELUMLP(torch.nn.Module):
@@ -664,13 +703,20 @@ class MinGRUMixer(torch.nn.Module):
 
 
 class RoutedExperts(torch.nn.Module):
-    """Mixture of feed-forward experts W_down relu(W_up h)^2 without biases.
-    The router (fp32) scores all its outputs with a softmax; the `top`
-    outputs with the largest corrected scores are chosen, among the `keep`
-    best of `groups` equal groups of neighbouring outputs; the chosen ones
-    weigh in with their uncorrected score times `scale`. The last `identity`
-    router outputs are identity experts (output = input). A shared expert of
-    the same form, when present, runs for every token.
+    """Mixture of feed-forward experts without biases, W_down relu(W_up h)^2
+    or, with `glu`, W_down (silu(W_gate h) * W_up h). The router is fp32.
+
+    route = "corrected_softmax": all router outputs are scored with a
+    softmax; the `top` outputs with the largest corrected scores are chosen,
+    among the `keep` best of `groups` equal groups of neighbouring outputs;
+    the chosen ones weigh in with their uncorrected score times `scale`.
+    route = "topk_logits": the `top` largest logits (router product plus a
+    bias) are chosen and weigh in with the softmax over the chosen logits.
+
+    The last `identity` router outputs are identity experts (output =
+    input). A shared expert of the same form, when present, runs for every
+    token; with `shared_gate` it is multiplied by sigmoid(w_sg . h), one
+    value per token (w_sg is kept as one more row of the router matrix).
 
     Chosen (token, expert) pairs get a row of a gathered batch - expert e
     owns rows base[e] + rank - so that each expert is one GEMM over its
@@ -681,36 +727,60 @@ class RoutedExperts(torch.nn.Module):
     PADDED_MAX_ROWS = 64
 
     def __init__(self, width, experts, ff, top, scale, identity, groups, keep,
-                 shared_ff, init):
+                 shared_ff, init, glu=False, route="corrected_softmax",
+                 shared_gate=False):
         super().__init__()
         n = experts + identity
+        if route not in ("corrected_softmax", "topk_logits"):
+            raise ValueError(f"unknown router {route!r}")
         if n % groups or not 1 <= keep <= groups:
             raise ValueError("router outputs must divide into their groups")
         if top > keep * (n // groups):
             raise ValueError("more experts per token than the kept groups hold")
+        if shared_gate and (route != "topk_logits" or not shared_ff):
+            raise ValueError("a gated shared expert needs the logit router "
+                             "and a shared expert")
         self.W, self.E, self.n, self.ff = width, experts, n, ff
         self.top, self.scale = top, scale
         self.groups, self.keep = groups, keep
+        self.glu, self.route, self.shared_gate = glu, route, shared_gate
+        self.act = sops.silu_glu if glu else sops.relu_squared
+        up = 2 * ff if glu else ff
         f32 = dict(dtype=torch.float32, device=init.device)
-        self.router = (torch.randn(n, width, generator=init.gen)
+        self.router = (torch.randn(n + (1 if shared_gate else 0), width,
+                                   generator=init.gen)
                        * width ** -0.5).to(**f32)
+        # per-output constant: correction of the choice, or logit bias
         self.correction = init.vec(n, -0.05, 0.05)
-        self.w_up = torch.stack([init.mat(ff, width) for _ in range(experts)])
+        self.w_up = torch.stack([init.mat(up, width) for _ in range(experts)])
         self.w_down = torch.stack([init.mat(width, ff) for _ in range(experts)])
         self.shared_up = self.shared_down = None
         if shared_ff:
-            self.shared_up = init.mat(shared_ff, width)
+            self.shared_up = init.mat(2 * shared_ff if glu else shared_ff,
+                                      width)
             self.shared_down = init.mat(width, shared_ff)
         self._pad_base = {}
 
+    def _up_rows(self, get, prefix):
+        if self.glu:      # fused rows: gate | up
+            return torch.cat([get(prefix + "gate"), get(prefix + "up")], 0)
+        return get(prefix + "up")
+
     def load(self, get: Getter):
-        _put(self.router, get("router"))
-        _put(self.correction, get("correction"))
-        _put(self.w_up, torch.stack([get(f"e{e}.up") for e in range(self.E)]))
+        if self.route == "topk_logits":
+            rows = [get("router")] + ([get("shared.sg").reshape(1, -1)]
+                                      if self.shared_gate else [])
+            _put(self.router, torch.cat(rows, 0))
+            _put(self.correction, get("router.b"))
+        else:
+            _put(self.router, get("router"))
+            _put(self.correction, get("correction"))
+        _put(self.w_up, torch.stack([self._up_rows(get, f"e{e}.")
+                                     for e in range(self.E)]))
         _put(self.w_down,
              torch.stack([get(f"e{e}.down") for e in range(self.E)]))
         if self.shared_up is not None:
-            _put(self.shared_up, get("shared.up"))
+            _put(self.shared_up, self._up_rows(get, "shared."))
             _put(self.shared_down, get("shared.down"))
 
     def _padded_base(self, cap, device):
@@ -722,16 +792,24 @@ class RoutedExperts(torch.nn.Module):
 
     def forward(self, h):
         T, E = h.shape[0], self.E
-        idx, wgt = sops.moe_route_rows(h, self.router, self.correction,
-                                       self.groups, self.keep, self.top,
-                                       self.scale)
+        sgate = None
+        if self.route == "topk_logits":
+            logits = F.linear(h.float(), self.router)
+            idx, wgt = sops.moe_route_topk(logits, self.n, self.correction,
+                                           self.top)
+            if self.shared_gate:
+                sgate = logits[:, self.n]
+        else:
+            idx, wgt = sops.moe_route_rows(h, self.router, self.correction,
+                                           self.groups, self.keep, self.top,
+                                           self.scale)
         rank, counts = sops.moe_dispatch(idx, self.n)
         if T <= self.PADDED_MAX_ROWS:
             # every expert gets a block of T rows: static shapes, no host read
             base = self._padded_base(T, h.device)
             xg = sops.moe_gather(h, idx, rank, base, E, E * T)
-            a = sops.relu_squared(torch.bmm(xg.view(E, T, self.W),
-                                            self.w_up.transpose(1, 2)))
+            a = self.act(torch.bmm(xg.view(E, T, self.W),
+                                   self.w_up.transpose(1, 2)))
             y = torch.bmm(a, self.w_down.transpose(1, 2)).view(E * T, self.W)
         else:
             cnt = counts[:E].tolist()
@@ -743,13 +821,192 @@ class RoutedExperts(torch.nn.Module):
             r0 = 0
             for e, n in enumerate(cnt):
                 if n:
-                    a = sops.relu_squared(F.linear(xg[r0:r0 + n],
-                                                   self.w_up[e]))
+                    a = self.act(F.linear(xg[r0:r0 + n], self.w_up[e]))
                     y[r0:r0 + n] = F.linear(a, self.w_down[e])
                 r0 += n
         shared = None
         if self.shared_up is not None:
-            shared = F.linear(sops.relu_squared(F.linear(h, self.shared_up)),
+            shared = F.linear(self.act(F.linear(h, self.shared_up)),
                               self.shared_down)
         return sops.moe_combine(y, h, idx, wgt, rank, base, E, shared,
-                                h.dtype)
+                                h.dtype, sgate)
+
+
+def distance_bias_table(rel: torch.Tensor, max_dist: int) -> torch.Tensor:
+    """fp32 [D + 1, H] from a bucketed table rel [B, H]: row n is the bias
+    of key distance n (the last row serves every distance >= D). Buckets:
+    n itself below B // 2; from there logarithmic steps that reach the last
+    bucket at distance D = max_dist:
+    min(B - 1, B//2 + floor(ln(n / (B//2)) / ln(D / (B//2)) * (B - B//2)))."""
+    import math
+    B = rel.shape[0]
+    half = B // 2
+    rows = []
+    for n in range(int(max_dist) + 1):
+        if n < half:
+            rows.append(n)
+        else:
+            rows.append(min(B - 1, half + int(math.floor(
+                math.log(n / half) / math.log(max_dist / half) * (B - half)))))
+    return rel.float()[torch.tensor(rows, dtype=torch.long,
+                                    device=rel.device)].contiguous()
+
+
+class CappedAttention(torch.nn.Module):
+    """Grouped-query softmax attention without rotation, with biases on
+    q, k, v and the output projection. q and k are RMS-normed over their
+    whole projection (all heads at once, one weight per entry) before being
+    split into heads; keys are cached normed. Options: a query temperature
+    1 + coef ln(floor((p + 1) / every) + 1), a soft cap c tanh(s / c) on the
+    scaled scores, and a learned bias by bucketed key distance (a table
+    [buckets, heads], see distance_bias_table) added after the cap. With
+    shared_cache the layer has no key/value projections and reads another
+    layer's cached keys and values with its own queries."""
+
+    def __init__(self, width, heads, kv_heads, dim, vdim, scale, eps, init,
+                 temp_coef=0.0, temp_every=1, softcap=0.0, buckets=0,
+                 bias_max=0, shared_cache=False):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("query heads must be a multiple of kv heads")
+        self.W, self.H, self.G, self.dk, self.dv = width, heads, kv_heads, dim, vdim
+        self.scale, self.eps = scale, eps
+        self.temp_coef, self.temp_every = float(temp_coef), int(temp_every)
+        self.softcap, self.bias_max = float(softcap or 0.0), int(bias_max)
+        self.shared_cache = shared_cache
+        self.nq = heads * dim
+        self.nk = 0 if shared_cache else kv_heads * dim
+        self.nv = 0 if shared_cache else kv_heads * vdim
+        self.off_k, self.off_v = self.nq, self.nq + self.nk
+        # fused rows: q | k | v, each with its bias
+        self.w_in = init.mat(self.off_v + self.nv, width)
+        self.b_in = init.vec(self.off_v + self.nv, -0.2, 0.2).to(init.dtype)
+        self.q_norm = init.vec(self.nq, 0.7, 1.3)
+        self.k_norm = None if shared_cache else init.vec(self.nk, 0.7, 1.3)
+        self.rel = init.vec((buckets, heads), -1.0, 1.0) if buckets else None
+        self.w_o = init.mat(width, heads * vdim)
+        self.b_o = init.vec(width, -0.2, 0.2).to(init.dtype)
+        self.refresh()
+
+    def refresh(self):
+        """The bias by distance from the bucket table."""
+        self.dist_bias = None
+        if self.rel is not None:
+            if not self.bias_max > self.rel.shape[0] // 2 >= 1:
+                raise ValueError("the distance bias needs at least two "
+                                 "buckets and a largest distance beyond the "
+                                 "exact ones")
+            self.dist_bias = distance_bias_table(self.rel, self.bias_max)
+
+    def state_shapes(self):
+        return []
+
+    def kv_shape(self):
+        return None if self.shared_cache else (self.G, self.dk, self.dv)
+
+    def load(self, get: Getter):
+        names = ["q"] + ([] if self.shared_cache else ["k", "v"])
+        _put(self.w_in, torch.cat([get(n) for n in names], 0))
+        _put(self.b_in, torch.cat([get(n + ".b") for n in names], 0))
+        _put(self.q_norm, get("q.norm"))
+        if not self.shared_cache:
+            _put(self.k_norm, get("k.norm"))
+        if self.rel is not None:
+            rel = get("rel")
+            if rel.shape != self.rel.shape:     # buckets come from the file
+                self.rel = torch.empty(rel.shape, dtype=self.rel.dtype,
+                                       device=self.rel.device)
+            _put(self.rel, rel)
+        _put(self.w_o, get("o"))
+        _put(self.b_o, get("o.b"))
+        self.refresh()
+
+    def forward(self, h, ctx: MixContext):
+        proj = F.linear(h, self.w_in, self.b_in)
+        own = not self.shared_cache
+        sops.rownorm_append(proj, self.nq, self.off_k, self.nk, self.off_v,
+                            self.nv, self.q_norm, self.k_norm, self.eps,
+                            ctx.kcache if own else None,
+                            ctx.vcache if own else None, ctx.slot_mapping)
+        y = sops.paged_attention_rows(
+            proj, 0, self.H, 1, ctx.kcache, ctx.vcache, self.dv,
+            ctx.positions, ctx.sb, self.scale, out_dtype=h.dtype,
+            temp_coef=self.temp_coef, temp_every=self.temp_every,
+            softcap=self.softcap, dist_bias=self.dist_bias)
+        return F.linear(y.view(h.shape[0], self.H * self.dv), self.w_o,
+                        self.b_o)
+
+
+class SSDMixer(torch.nn.Module):
+    """State-space mixer in the scalar-decay (state-space duality) form.
+    W_in h = z | x | B | C | dt with inner = heads * vdim channels for z
+    and x, groups * state for B and C, one dt per head. x, B, C pass a
+    short causal per-channel convolution with bias and SiLU. Per head
+    (sharing B, C with its group): dt = softplus(dt + dt_bias),
+    S <- exp(-exp(A_log) dt) S + dt B x^T (S is state x vdim),
+    y = S^T C + D x. Output: y * silu(z), RMS-normed in norm_groups equal
+    parts of the row, times a weight, then W_o. The decay, step size and
+    state are fp32."""
+
+    def __init__(self, width, heads, vdim, state, groups, norm_groups, conv,
+                 eps, init):
+        super().__init__()
+        inner = heads * vdim
+        if heads % groups or inner % norm_groups:
+            raise ValueError("heads must divide into groups, channels into "
+                             "norm groups")
+        self.W, self.H, self.P, self.N, self.G = width, heads, vdim, state, groups
+        self.inner, self.ng, self.taps, self.eps = inner, norm_groups, conv, eps
+        self.Cc = inner + 2 * groups * state
+        self.off_dt = inner + self.Cc
+        self.w_in = init.mat(self.off_dt + heads, width)
+        self.conv_w = init.vec((self.Cc, conv), -0.5, 0.8)
+        self.conv_b = init.vec(self.Cc, -0.2, 0.2)
+        self.dt_bias = init.vec(heads, -3.0, 0.0)
+        self.A_log = init.vec(heads, -1.0, 1.5)
+        self.D = init.vec(heads, 0.5, 1.5)
+        self.norm_w = init.vec(inner, 0.7, 1.3)
+        self.w_o = init.mat(width, inner)
+
+    def state_shapes(self):
+        return [(self.H, self.N, self.P), (self.taps - 1, self.Cc)]
+
+    def kv_shape(self):
+        return None
+
+    def load(self, get: Getter):
+        _put(self.w_in, get("in"))
+        _put(self.conv_w, get("conv"))
+        _put(self.conv_b, get("conv.b"))
+        _put(self.dt_bias, get("dt_bias"))
+        _put(self.A_log, get("A_log"))
+        _put(self.D, get("D"))
+        _put(self.norm_w, get("norm"))
+        _put(self.w_o, get("o"))
+
+    def forward(self, h, ctx: MixContext):
+        proj = F.linear(h, self.w_in)
+        S, conv_state = ctx.states
+        xbc = sops.causal_conv(proj[:, self.inner:], self.Cc, self.conv_w,
+                               self.conv_b, True, conv_state, ctx.sb)
+        y = sops.ssd_scan(xbc, proj[:, self.off_dt:], self.dt_bias, self.A_log,
+                          self.D, S, ctx.sb, self.H, self.P, self.N, self.G)
+        y = sops.gated_group_norm(y, proj, self.norm_w, self.ng, self.eps,
+                                  h.dtype)
+        return F.linear(y, self.w_o)
+
+
+class GeluMLP(torch.nn.Module):
+    """Dense feed-forward W_down gelu(W_up h) with the exact (erf) GELU."""
+
+    def __init__(self, width, ff, init):
+        super().__init__()
+        self.w_up = init.mat(ff, width)
+        self.w_down = init.mat(width, ff)
+
+    def load(self, get: Getter):
+        _put(self.w_up, get("up"))
+        _put(self.w_down, get("down"))
+
+    def forward(self, h):
+        return F.linear(sops.gelu_erf(F.linear(h, self.w_up)), self.w_down)

@@ -23,6 +23,9 @@ def build_model(cfg: ModelConfig, device, dtype, tp=None, seed: int = 0):
     if cfg.arch == "kefesun":
         from .kefesun import KefesunForCausalLM
         return KefesunForCausalLM(cfg, device, dtype, tp, seed)
+    if cfg.arch == "muzulorn":
+        from .muzulorn import MuzulornForCausalLM
+        return MuzulornForCausalLM(cfg, device, dtype, tp, seed)
     raise ValueError(f"unknown arch {cfg.arch}")
 
 
@@ -30,7 +33,8 @@ def build_model(cfg: ModelConfig, device, dtype, tp=None, seed: int = 0):
 # whose config_from_json reads them
 LAYER_LIST_ARCHS = {"bolatar": "dynamo_amd.models.bolatar",
                     "fironex": "dynamo_amd.models.fironex",
-                    "kefesun": "dynamo_amd.models.kefesun"}
+                    "kefesun": "dynamo_amd.models.kefesun",
+                    "muzulorn": "dynamo_amd.models.muzulorn"}
 
 
 def native_extensions(cfg: ModelConfig, device: str):

@@ -292,7 +292,9 @@ def latent_append(cache, z, z_col: int, norm_w, slot_mapping, positions,
 def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
                          dv: int, positions, sb: SeqBatch, scale: float,
                          window: int = 0, keep_first: int = 0, head_bias=None,
-                         sigmoid: bool = False, out_dtype=torch.float32):
+                         sigmoid: bool = False, out_dtype=torch.float32,
+                         temp_coef: float = 0.0, temp_every: int = 1,
+                         softcap: float = 0.0, dist_bias=None, sink=None):
     """Causal attention of every row over its sequence's pages.
     -> [T, H, kmaps, dv] (fp32 unless out_dtype says otherwise). Queries lie
     in q at off_q as [H][kmaps][dk]; kcache [P, G, ps, kmaps * dk]; values
@@ -301,7 +303,12 @@ def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
     and also the keys j < keep_first whatever their distance. head_bias
     (fp32 [H]) is added to the scaled scores. The weights are a softmax over
     the visible keys, or with `sigmoid` the plain sigmoid of each score
-    (not normalised over the keys)."""
+    (not normalised over the keys). Further options of the softmax form: a
+    query temperature 1 + temp_coef ln(floor((i + 1) / temp_every) + 1) on
+    the scaled scores, a soft cap c tanh(score / c) after it, a bias by
+    distance dist_bias[min(i - j, D), h] (fp32 [D + 1, H]) added after the
+    cap, and a per-head sink (fp32 [H]): exp(sink_h) joins the softmax
+    denominator without a key or value."""
     if q.is_cuda:
         T = q.shape[0]
         out = torch.empty(T, H, kmaps, dv, dtype=out_dtype, device=q.device)
@@ -319,7 +326,9 @@ def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
         tiled = fits and sb.tiles is not None
         ndec = min(sb.num_decode, T)
         done = 0
-        opts = (int(window), int(keep_first), head_bias, bool(sigmoid))
+        opts = (int(window), int(keep_first), head_bias, bool(sigmoid),
+                float(softcap), dist_bias, sink)
+        temp = (float(temp_coef), int(temp_every))
         if (fits and ndec and H // G >= 8 and f32out
                 and m.paged_attention_mfma_supported(krow // kmaps, dv, True)):
             nsplit = max(1, min(16, 512 // (ndec * G * kmaps)))
@@ -328,24 +337,25 @@ def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
             m.paged_attention_mfma_decode(
                 out[:ndec], part, q[:ndec], off_q, kcache, vcache,
                 sb.page_table, sb.tok_seq[:ndec], positions[:ndec],
-                sb.seq_len, float(scale), int(kmaps), *opts)
+                sb.seq_len, float(scale), *temp, int(kmaps), *opts)
             done = ndec
         end = ndec if tiled else T
         if end > done:
             m.paged_attention_rows(
                 out[done:end], q[done:end], off_q, kcache, vcache,
                 sb.page_table, sb.tok_seq[done:end], positions[done:end],
-                sb.seq_len, None, None, float(scale), 0.0, 1, int(kmaps),
+                sb.seq_len, None, None, float(scale), *temp, int(kmaps),
                 *opts)
         if tiled and sb.tiles[0].numel():
             m.paged_attention_mfma(
                 out, q, off_q, kcache, vcache, sb.page_table, sb.tiles[0],
                 sb.tiles[1], 64, sb.tok_seq, positions, None, None,
-                float(scale), 0.0, 1, int(kmaps), *opts)
+                float(scale), *temp, int(kmaps), *opts)
         return out
     return seq_ref.paged_attention_rows(
         q, off_q, H, kmaps, kcache, vcache, dv, positions, sb, scale, window,
-        keep_first, head_bias, sigmoid).to(out_dtype)
+        keep_first, head_bias, sigmoid, temp_coef, temp_every, softcap,
+        dist_bias, sink).to(out_dtype)
 
 
 def diff_norm_gate(a, lam, post: float, gate, eps: float, out_dtype):
@@ -537,12 +547,164 @@ def moe_gather(h, idx, rank, base, E: int, rows: int):
     return seq_ref.moe_gather(h, idx, rank, base, E, rows)
 
 
-def moe_combine(y, h, idx, wgt, rank, base, E: int, shared, out_dtype):
+def moe_combine(y, h, idx, wgt, rank, base, E: int, shared, out_dtype,
+                shared_gate=None):
     """out[t] = sum_j wgt[t, j] * (y[base[e] + rank[t, j]] if e < E else
-    h[t]) (+ shared[t]), summed in fp32 in the order of j."""
+    h[t]) (+ shared[t], times sigmoid(shared_gate[t]) when a raw gate value
+    per token is given), summed in fp32 in the order of j."""
     if h.is_cuda:
         out = torch.empty(h.shape, dtype=out_dtype, device=h.device)
-        hip_seq().moe_combine(out, y, h, idx, wgt, rank, base, int(E), shared)
+        hip_seq().moe_combine(out, y, h, idx, wgt, rank, base, int(E), shared,
+                              shared_gate)
         return out
     return seq_ref.moe_combine(y, h, idx, wgt, rank, base, E, shared,
+                               out_dtype, shared_gate)
+
+
+# -- hashed pair embedding, stream mixing, whole-projection norms, state-space
+# -- scan, grouped gated norm, top-k router over logits -----------------------
+def embed_pair_hash(ids, embed, table, mul_prev: int, mul_cur: int,
+                    prev_state, sb: SeqBatch):
+    """fp32 [T, W]: embed[id] + table[(prev * mul_prev + id * mul_cur) mod n]
+    with n = rows of table - 1; a sequence's first token takes row n. The
+    previous token of a portion's first row comes from prev_state
+    (fp32 [slots, 1], the token id as a number), which is left holding the
+    portion's last token."""
+    if embed.is_cuda:
+        out = torch.empty(ids.shape[0], embed.shape[1], dtype=torch.float32,
+                          device=embed.device)
+        hip_seq().embed_pair_hash(out, ids, embed, table, int(mul_prev),
+                                  int(mul_cur), prev_state, sb.tok_seq,
+                                  *_args(sb))
+        return out
+    return seq_ref.embed_pair_hash(ids, embed, table, mul_prev, mul_cur,
+                                   prev_state, sb)
+
+
+def stream_step(xs, delta, mix, out_w, mult: float, in_w, norm_w, eps: float,
+                out_dtype):
+    """One step on S parallel residual streams xs (fp32 [T, S, W], in
+    place). With delta (a sublayer's output): every stream t becomes
+    sum_s mix[s, t] xs[s] + mult * out_w[t] * delta, all from the old
+    streams. Then, with in_w: the read u = sum_s in_w[s] xs[s] is returned
+    RMS-normed times (1 + norm_w) in out_dtype, or - without norm_w - as it
+    is in fp32. mix fp32 [S, S], out_w / in_w fp32 [S]."""
+    if xs.is_cuda:
+        T, S, W = xs.shape
+        out = None
+        if in_w is not None:
+            out = torch.empty(T, W, device=xs.device,
+                              dtype=out_dtype if norm_w is not None
+                              else torch.float32)
+        hip_seq().stream_step(out, xs, delta, mix, out_w, float(mult), in_w,
+                              norm_w, float(eps))
+        return out
+    return seq_ref.stream_step(xs, delta, mix, out_w, mult, in_w, norm_w, eps,
                                out_dtype)
+
+
+def rms_norm_cols(x, col: int, n: int, w, eps: float, out_dtype):
+    """[T, n]: columns [col, col + n) of x divided by their root mean
+    square, times w (fp32 [n])."""
+    if x.is_cuda:
+        out = torch.empty(x.shape[0], n, dtype=out_dtype, device=x.device)
+        hip_seq().rms_norm_cols(out, x, int(col), w, float(eps))
+        return out
+    return seq_ref.rms_norm_cols(x, col, n, w, eps, out_dtype)
+
+
+def rownorm_append(proj, nq: int, off_k: int, nk: int, off_v: int, nv: int,
+                   qw, kw, eps: float, kcache, vcache, slot_mapping):
+    """Per token row of proj: the whole query run [0, nq) is divided by its
+    root mean square and multiplied by qw (fp32 [nq]) in place; with caches,
+    the whole key run [off_k, off_k + nk) likewise with kw, written with the
+    raw values [off_v, off_v + nv) to the token's cache slot (kcache
+    [P, G, ps, nk / G], vcache [P, G, ps, nv / G])."""
+    if proj.is_cuda:
+        hip_seq().rownorm_append(proj, int(nq), int(off_k), int(nk),
+                                 int(off_v), int(nv), qw, kw, float(eps),
+                                 kcache, vcache, slot_mapping)
+    else:
+        seq_ref.rownorm_append(proj, nq, off_k, nk, off_v, nv, qw, kw, eps,
+                               kcache, vcache, slot_mapping)
+
+
+def heads_major(x, out_dtype):
+    """x [T, H, R] -> [H, T, R] in out_dtype (the layout a per-head batched
+    product reads)."""
+    if x.is_cuda:
+        T, H, R = x.shape
+        out = torch.empty(H, T, R, dtype=out_dtype, device=x.device)
+        hip_seq().heads_major(out, x)
+        return out
+    return seq_ref.heads_major(x, out_dtype)
+
+
+def heads_gate(o, gate, out_dtype):
+    """o [H, T, dv] (head-major), gate [T, >= H*dv] -> [T, H*dv] =
+    o * sigmoid(gate), element by element."""
+    if o.is_cuda:
+        H, T, dv = o.shape
+        out = torch.empty(T, H * dv, dtype=out_dtype, device=o.device)
+        hip_seq().heads_gate(out, o, gate)
+        return out
+    return seq_ref.heads_gate(o, gate, out_dtype)
+
+
+def ssd_scan(xbc, dt_raw, dt_bias, A_log, D, state, sb: SeqBatch, H: int,
+             P: int, N: int, G: int):
+    """State-space recurrence over fp32 xbc [T, H*P + 2*G*N] = x | B | C:
+    per head h (group h // (H / G)), dt = softplus(dt_raw + dt_bias),
+    S <- exp(-exp(A_log) dt) S + dt B x^T, y = S^T C + D x.
+    state fp32 [slots, H, N, P]; dt_raw [T, H] (any row stride).
+    -> fp32 [T, H*P]."""
+    if xbc.is_cuda:
+        out = torch.empty(xbc.shape[0], H * P, dtype=torch.float32,
+                          device=xbc.device)
+        hip_seq().ssd_scan(out, xbc, dt_raw, dt_bias, A_log, D, state,
+                           *_args(sb), int(G))
+        return out
+    return seq_ref.ssd_scan(xbc, dt_raw, dt_bias, A_log, D, state, sb, H, P,
+                            N, G)
+
+
+def gated_group_norm(y, z, w, groups: int, eps: float, out_dtype):
+    """fp32 y [T, C] times silu(z[:, :C]), RMS-normed in `groups` equal
+    parts of the row, times w (fp32 [C])."""
+    if y.is_cuda:
+        out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
+        hip_seq().gated_group_norm(out, y, z, w, int(groups), float(eps))
+        return out
+    return seq_ref.gated_group_norm(y, z, w, groups, eps, out_dtype)
+
+
+def gelu_erf(x):
+    if x.is_cuda:
+        out = torch.empty_like(x)
+        hip_seq().gelu_erf(out, x)
+        return out
+    return seq_ref.gelu_erf(x)
+
+
+def silu_glu(gate_up):
+    """[..., 2F] (gate | up) -> silu(gate) * up."""
+    if gate_up.is_cuda:
+        Fd = gate_up.shape[-1] // 2
+        out = torch.empty(*gate_up.shape[:-1], Fd, dtype=gate_up.dtype,
+                          device=gate_up.device)
+        hip_seq().silu_glu(out.view(-1, Fd), gate_up.view(-1, 2 * Fd))
+        return out
+    return seq_ref.silu_glu(gate_up)
+
+
+def moe_route_topk(logits, n: int, bias, top: int):
+    """Router that keeps the `top` largest of the first n columns of the
+    fp32 logits (+ bias fp32 [n]); the weights are the softmax over the
+    chosen ones only. -> (int32 [T, top], fp32 [T, top])."""
+    if logits.is_cuda:
+        T = logits.shape[0]
+        idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+        wgt = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+        hip_seq().moe_route_topk(idx, wgt, logits, int(n), bias)
+        return idx, wgt
+    return seq_ref.moe_route_topk(logits, n, bias, top)

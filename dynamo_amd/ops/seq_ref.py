@@ -304,7 +304,8 @@ def latent_append(cache, z, z_col, norm_w, slot_mapping, positions, freqs,
 
 def paged_attention_rows(q, off_q, H, kmaps, kcache, vcache, dv, positions, sb,
                          scale, window, keep_first=0, head_bias=None,
-                         sigmoid=False):
+                         sigmoid=False, temp_coef=0.0, temp_every=1,
+                         softcap=0.0, dist_bias=None, sink=None):
     """fp32 [T, H, kmaps, dv]; see ops.seq.paged_attention_rows."""
     P, G, ps, krow = kcache.shape
     dk = krow // kmaps
@@ -332,11 +333,24 @@ def paged_attention_rows(q, off_q, H, kmaps, kcache, vcache, dv, positions, sb,
             i = pos[t]
             j = torch.arange(i + 1)
             seen = ((i - j < window) | (j < keep_first)) if window else j >= 0
-            s = torch.einsum("hmd,hjmd->hmj", qq[t] * scale, kk[:, :i + 1])
+            temp = 1.0
+            if temp_coef != 0.0:
+                temp += temp_coef * math.log((i + 1) // temp_every + 1)
+            s = torch.einsum("hmd,hjmd->hmj", qq[t] * (temp * scale),
+                             kk[:, :i + 1])
+            if softcap:
+                s = softcap * torch.tanh(s / softcap)
+            if dist_bias is not None:
+                dist = (i - j).clamp(max=dist_bias.shape[0] - 1)
+                s = s + dist_bias[dist].t().view(H, 1, i + 1)
             if head_bias is not None:
                 s = s + head_bias.view(H, 1, 1)
             if sigmoid:
                 wgt = torch.sigmoid(s) * seen
+            elif sink is not None:
+                s = s.masked_fill(~seen, float("-inf"))
+                full = torch.cat([s, sink.view(H, 1, 1).expand(H, kmaps, 1)], -1)
+                wgt = torch.softmax(full, -1)[..., :-1]
             else:
                 wgt = torch.softmax(s.masked_fill(~seen, float("-inf")), -1)
             out[t] = torch.einsum("hmj,hjd->hmd", wgt, vv[:, :i + 1])
@@ -499,7 +513,8 @@ def moe_gather(h, idx, rank, base, E, rows):
     return xg
 
 
-def moe_combine(y, h, idx, wgt, rank, base, E, shared, out_dtype):
+def moe_combine(y, h, idx, wgt, rank, base, E, shared, out_dtype,
+                shared_gate=None):
     T, k = idx.shape
     out = torch.zeros(T, h.shape[1], dtype=torch.float32)
     hf = h.float()
@@ -510,5 +525,143 @@ def moe_combine(y, h, idx, wgt, rank, base, E, shared, out_dtype):
                    else hf[t])
             out[t] += wgt[t, j] * src
     if shared is not None:
-        out += shared.float()
+        sh = shared.float()
+        if shared_gate is not None:     # one raw gate value per token
+            sh = sh * torch.sigmoid(shared_gate.float()).view(T, 1)
+        out += sh
     return out.to(out_dtype)
+
+
+# -- hashed pair embedding, stream mixing, whole-projection norms, state-space
+# -- scan, grouped gated norm, top-k router over logits -----------------------
+def embed_pair_hash(ids, embed, table, mul_prev, mul_cur, prev_state, sb):
+    """fp32 [T, W]: embed[id] + table[(prev * mul_prev + id * mul_cur) mod n],
+    n = rows of table - 1; a sequence's first token takes row n. The last
+    token of each portion is left in prev_state[slot] for the next one."""
+    x = embed[ids.long()].float()
+    n = table.shape[0] - 1
+    tok = ids.long()
+    rows = torch.empty_like(tok)
+    for start, cnt, slot, pos0 in sb.spans():
+        if cnt == 0:
+            continue
+        prev = torch.empty(cnt, dtype=torch.long)
+        prev[1:] = tok[start:start + cnt - 1]
+        prev[0] = int(prev_state[slot, 0]) if pos0 > 0 else 0
+        r = (prev * mul_prev + tok[start:start + cnt] * mul_cur) % n
+        if pos0 == 0:
+            r[0] = n
+        rows[start:start + cnt] = r
+        prev_state[slot, 0] = float(tok[start + cnt - 1])
+    return x + table[rows].float()
+
+
+def stream_step(xs, delta, mix, out_w, mult, in_w, norm_w, eps, out_dtype):
+    """xs fp32 [T, S, W], in place: with delta, stream t becomes
+    sum_s mix[s, t] xs[s] + mult * out_w[t] * delta. Then, with in_w, returns
+    the read u = sum_s in_w[s] xs[s] RMS-normed times (1 + norm_w) in
+    out_dtype (u itself in fp32 without norm_w)."""
+    if delta is not None:
+        new = torch.einsum("st,nsw->ntw", mix.float(), xs) \
+            + mult * out_w.float()[None, :, None] * delta.float()[:, None, :]
+        xs.copy_(new)
+    if in_w is None:
+        return None
+    u = torch.einsum("s,nsw->nw", in_w.float(), xs)
+    if norm_w is None:
+        return u
+    u = u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps)
+    return (u * (1.0 + norm_w.float())).to(out_dtype)
+
+
+def rms_norm_cols(x, col, n, w, eps, out_dtype):
+    v = x[:, col:col + n].float()
+    v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    return (v * w.float()).to(out_dtype)
+
+
+def rownorm_append(proj, nq, off_k, nk, off_v, nv, qw, kw, eps, kcache,
+                   vcache, slot_mapping):
+    T = proj.shape[0]
+    q = rms_norm_cols(proj, 0, nq, qw, eps, proj.dtype)
+    proj[:, :nq] = q
+    if kcache is None:
+        return
+    P, G, ps, dk = kcache.shape
+    dv = vcache.shape[3]
+    k = rms_norm_cols(proj, off_k, nk, kw, eps, kcache.dtype).view(T, G, dk)
+    v = proj[:, off_v:off_v + nv].view(T, G, dv)
+    for t, slot in enumerate(slot_mapping.tolist()):
+        if slot < 0:
+            continue
+        kcache[slot // ps, :, slot % ps] = k[t]
+        vcache[slot // ps, :, slot % ps] = v[t]
+
+
+def heads_gate(o, gate, out_dtype):
+    """o [H, T, dv], gate [T, >= H*dv] -> [T, H*dv] = o * sigmoid(gate)."""
+    H, T, dv = o.shape
+    y = o.float().transpose(0, 1).reshape(T, H * dv)
+    return (y * torch.sigmoid(gate[:, :H * dv].float())).to(out_dtype)
+
+
+def heads_major(x, out_dtype):
+    """x [T, H, R] -> [H, T, R] in out_dtype."""
+    return x.transpose(0, 1).contiguous().to(out_dtype)
+
+
+def ssd_scan(xbc, dt_raw, dt_bias, A_log, D, state, sb, H, P, N, G):
+    """State-space recurrence per head over fp32 xbc [T, H*P + 2*G*N] =
+    x | B | C (after convolution and activation):
+    dt = softplus(dt_raw + dt_bias); S <- exp(-exp(A_log) dt) S + dt B x^T;
+    y = S^T C + D x. state fp32 [slots, H, N, P]. -> fp32 [T, H*P]."""
+    T = xbc.shape[0]
+    inner = H * P
+    x = xbc[:, :inner].view(T, H, P)
+    Bm = xbc[:, inner:inner + G * N].view(T, G, N)
+    Cm = xbc[:, inner + G * N:inner + 2 * G * N].view(T, G, N)
+    rep = H // G
+    dt = F.softplus(dt_raw.float() + dt_bias, threshold=20.0)      # [T, H]
+    decay = torch.exp(-torch.exp(A_log) * dt)
+    out = torch.empty(T, H, P, dtype=torch.float32)
+    for start, n, slot, pos0 in sb.spans():
+        if n == 0:
+            continue
+        S = state[slot].clone() if pos0 > 0 else torch.zeros_like(state[slot])
+        for t in range(start, start + n):
+            Bt = Bm[t].repeat_interleave(rep, 0)                   # [H, N]
+            Ct = Cm[t].repeat_interleave(rep, 0)
+            S = decay[t].view(H, 1, 1) * S + \
+                (dt[t].view(H, 1) * Bt).unsqueeze(2) * x[t].unsqueeze(1)
+            out[t] = torch.einsum("hnp,hn->hp", S, Ct) + D.view(H, 1) * x[t]
+        state[slot] = S
+    return out.view(T, inner)
+
+
+def gated_group_norm(y, z, w, groups, eps, out_dtype):
+    """(y * silu(z)) RMS-normed in `groups` equal parts, times w."""
+    T, C = y.shape
+    v = y.float() * F.silu(z[:, :C].float())
+    v = v.view(T, groups, C // groups)
+    v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps)
+    return (v.reshape(T, C) * w.float()).to(out_dtype)
+
+
+def gelu_erf(x):
+    return F.gelu(x.float()).to(x.dtype)
+
+
+def silu_glu(gate_up):
+    Fd = gate_up.shape[-1] // 2
+    g, u = gate_up[..., :Fd].float(), gate_up[..., Fd:].float()
+    return (F.silu(g) * u).to(gate_up.dtype)
+
+
+def moe_route_topk(logits, n, bias, top):
+    """The `top` largest of the first n columns of logits (+ bias); weights
+    are the softmax over the chosen ones only."""
+    z = logits[:, :n].float()
+    if bias is not None:
+        z = z + bias
+    val, idx = z.topk(top, -1)
+    return idx.to(torch.int32), torch.softmax(val, -1)
