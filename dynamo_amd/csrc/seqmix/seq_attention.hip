@@ -23,7 +23,11 @@
 // `keep_first` keys of a sequence may stay visible whatever their distance;
 // a per-head constant may be added to the scaled scores; and the weights
 // may be plain sigmoids of the scores (not normalised over the keys)
-// instead of a softmax.
+// instead of a softmax. The softmax form further takes a soft cap
+// c tanh(score / c) on the scaled scores, a bias looked up by key distance
+// in a table [dist_max + 1, H] (added after the cap; distances beyond the
+// table take its last row), and a per-head sink: exp(sink_h) is added to the
+// softmax denominator, with no key and no value.
 #include "seq_common.h"
 
 namespace {
@@ -104,7 +108,8 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
     const float* __restrict__ r2, int H, int G, int dk, int dv, int ps,
     float scale, float temp_coef, int temp_every, int has_bias, int kmaps,
     int vrow, int window, int keep_first, const float* __restrict__ head_bias,
-    int sigmoid) {
+    int sigmoid, float softcap, const float* __restrict__ dist_bias,
+    int dist_max, const float* __restrict__ sink) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // q [GS][dk]; merge [waves][GS][2 + dv]
   constexpr int VN = Vec16<T>::N;
@@ -212,7 +217,9 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
         float x = d[a];
         x += __shfl_xor(x, 1, 64);
         x += __shfl_xor(x, 2, 64);
+        if (softcap > 0.f) x = softcap * tanhf(x / softcap);
         if (has_bias) x -= b1[a] * log1pf(b2[a] * (float)(pos - jc));
+        if (dist_bias) x += dist_bias[min(pos - jc, dist_max) * H + h0 + a];
         x += hb[a];
         sc[p][a] = (j < ctx && (j >= jmin || j < keep_first)) ? x : -INFINITY;
       }
@@ -338,9 +345,9 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
       }
       continue;
     }
-    float mx = -INFINITY;
+    float mx = sink ? sink[h0 + a] : -INFINITY;
     for (int w = 0; w < nwv; w++) mx = fmaxf(mx, mg[(w * GS + a) * MS]);
-    float lt = 0.f;
+    float lt = sink ? expf(sink[h0 + a] - mx) : 0.f;
     for (int w = 0; w < nwv; w++) {
       const float mw = mg[(w * GS + a) * MS];
       if (mw != -INFINITY) lt += expf(mw - mx) * mg[(w * GS + a) * MS + 1];
@@ -367,7 +374,9 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
                       c10::optional<torch::Tensor>& r2, double scale,
                       double temp_coef, int64_t temp_every, int kmaps,
                       int window, int keep_first,
-                      c10::optional<torch::Tensor>& head_bias, bool sigmoid) {
+                      c10::optional<torch::Tensor>& head_bias, bool sigmoid,
+                      double softcap, c10::optional<torch::Tensor>& dist_bias,
+                      c10::optional<torch::Tensor>& sink) {
   const int T_ = out.size(0), H = out.size(1);
   const int G = kcache.size(1), ps = kcache.size(2);
   const int dk = kcache.size(3) / kmaps;
@@ -404,7 +413,10 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
       r1 ? cptr<float>(*r1) : nullptr, r2 ? cptr<float>(*r2) : nullptr, H,  \
       G, dk, dv, ps, (float)scale, (float)temp_coef, (int)temp_every,       \
       r1 ? 1 : 0, kmaps, vrow, window, keep_first,                          \
-      head_bias ? cptr<float>(*head_bias) : nullptr, sigmoid ? 1 : 0)
+      head_bias ? cptr<float>(*head_bias) : nullptr, sigmoid ? 1 : 0,       \
+      (float)softcap, dist_bias ? cptr<float>(*dist_bias) : nullptr,        \
+      dist_bias ? (int)dist_bias->size(0) - 1 : 0,                          \
+      sink ? cptr<float>(*sink) : nullptr)
 #define LAUNCH_GS(GS_)                                                      \
   do {                                                                      \
     if (vec && small) LAUNCH_ATT(GS_, true, 2);                             \
@@ -462,9 +474,21 @@ void paged_attention_rows(torch::Tensor out, torch::Tensor proj, int64_t off_q,
                           double temp_coef, int64_t temp_every, int64_t kmaps,
                           int64_t window, int64_t keep_first,
                           c10::optional<torch::Tensor> head_bias,
-                          bool sigmoid) {
+                          bool sigmoid, double softcap,
+                          c10::optional<torch::Tensor> dist_bias,
+                          c10::optional<torch::Tensor> sink) {
   SEQ_CHECK(out.dim() == 4 && out.is_contiguous() && out.size(2) == kmaps,
             "attention out [T, H, maps, dv]");
+  SEQ_CHECK(softcap >= 0.0 && !(sigmoid && (sink || softcap > 0.0)),
+            "soft cap / sink belong to the softmax form");
+  if (dist_bias)
+    SEQ_CHECK(dist_bias->scalar_type() == torch::kFloat &&
+                  dist_bias->is_contiguous() && dist_bias->dim() == 2 &&
+                  dist_bias->size(0) >= 1 && dist_bias->size(1) == out.size(1),
+              "distance bias fp32 [D + 1, H]");
+  if (sink)
+    SEQ_CHECK(sink->scalar_type() == torch::kFloat && sink->is_contiguous() &&
+                  sink->numel() == out.size(1), "sink fp32 [H]");
   SEQ_CHECK(keep_first >= 0, "kept first keys");
   if (head_bias)
     SEQ_CHECK(head_bias->scalar_type() == torch::kFloat &&
@@ -520,12 +544,13 @@ void paged_attention_rows(torch::Tensor out, torch::Tensor proj, int64_t off_q,
                                  page_table, tok_seq, positions, seq_len, r1,
                                  r2, scale, temp_coef, temp_every, (int)kmaps,
                                  (int)window, (int)keep_first, head_bias,
-                                 sigmoid);
+                                 sigmoid, softcap, dist_bias, sink);
     else
       launch_attention<T, T>(out, proj, off_q, kcache, vptr, dv, vrow,
                              page_table, tok_seq, positions, seq_len, r1, r2,
                              scale, temp_coef, temp_every, (int)kmaps,
-                             (int)window, (int)keep_first, head_bias, sigmoid);
+                             (int)window, (int)keep_first, head_bias, sigmoid,
+                             softcap, dist_bias, sink);
   });
 }
 
@@ -540,5 +565,6 @@ void biased_attention(torch::Tensor out, torch::Tensor proj, int64_t off_q,
                 out.scalar_type() == proj.scalar_type(), "attention out");
   paged_attention_rows(out.unsqueeze(2), proj, off_q, kcache, vcache,
                        page_table, tok_seq, positions, seq_len, r1, r2, scale,
-                       temp_coef, temp_every, 1, 0, 0, c10::nullopt, false);
+                       temp_coef, temp_every, 1, 0, 0, c10::nullopt, false, 0.0,
+                       c10::nullopt, c10::nullopt);
 }

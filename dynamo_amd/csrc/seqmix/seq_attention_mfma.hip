@@ -5,7 +5,9 @@
 // maps per kv head, values that alias the head of the key rows (latent
 // attention), fp32 output, kept first keys under a window, a per-head
 // constant on the scores, and plain sigmoid weights (not normalised over
-// the keys) in place of the softmax.
+// the keys) in place of the softmax; for the softmax form also a soft cap
+// on the scaled scores, a bias by key distance from a table, and a per-head
+// sink in the denominator.
 //
 // A workgroup (4 waves) owns a tile of up to 64 consecutive rows of one
 // sequence and one (query head, key map); each wave owns 16 rows. Keys and
@@ -75,6 +77,7 @@ struct MfmaArgs {
   float scale, temp_coef; int temp_every, has_bias;
   int kmaps, krow, vrow, window;
   int keep_first; const float* head_bias; int sigmoid;
+  float softcap; const float* dist_bias; int dist_max; const float* sink;
   // HEADS mode: rows of a tile are heads of one decoded token
   const int* seq_len; int nsplit; float* partial;
 };
@@ -165,6 +168,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const float my_hb = !a.head_bias ? 0.f
                       : HEADS ? (my_ok ? a.head_bias[h + my_row] : 0.f)
                               : a.head_bias[h];
+  // head of this lane's row, for the tables indexed by head
+  const int my_head = HEADS ? h + (my_ok ? my_row : 0) : h;
+  const float* my_dist = a.dist_bias ? a.dist_bias + my_head : nullptr;
   // prompt rows are in order; the heads of a token share its position
   const int kv_end = a.positions[HEADS ? row0 : row0 + nrows - 1] + 1;
   // the first key any row of the tile sees
@@ -348,8 +354,11 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
 #pragma unroll
         for (int r = 0; r < 4; r++) {
           const int j = t0 + n * 16 + lg * 4 + r;
-          float x = s[n][r] * my_qmul + my_hb;
+          float x = s[n][r] * my_qmul;
+          if (a.softcap > 0.f) x = a.softcap * tanhf(x / a.softcap);
+          x += my_hb;
           if (a.has_bias) x -= b1 * log1pf(b2 * (float)max(my_pos - j, 0));
+          if (my_dist) x += my_dist[min(max(my_pos - j, 0), a.dist_max) * H];
           const bool seen = j <= my_pos && (window == 0 || j > my_pos - window ||
                                             j < a.keep_first);
           x = seen ? x : -INFINITY;
@@ -446,7 +455,13 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     return;
   }
   // ---- normalise and store query row lr, channels 16 d + 4 lg + r
-  const float inv = a.sigmoid ? 1.f : 1.f / l;
+  float inv = a.sigmoid ? 1.f : 1.f / l;
+  if (a.sink) {  // exp(sink) joins the denominator
+    const float sk = a.sink[my_head];
+    const float mm = fmaxf(m, sk);
+    const float c = expf(m - mm);
+    inv = c / (l * c + expf(sk - mm));
+  }
   TO* o = out + (((int64_t)(row0 + my_row) * H + h) * a.kmaps + map) * dv;
 #pragma unroll
   for (int d = 0; d < DN; d++)
@@ -465,19 +480,22 @@ __global__ void merge_splits_kernel(float* __restrict__ out,
                                     const float* __restrict__ partial,
                                     const int* __restrict__ tok_seq,
                                     const int* __restrict__ seq_len,
-                                    int HM, int nsplit, int dv, int plain_sum) {
+                                    int HM, int nsplit, int dv, int plain_sum,
+                                    const float* __restrict__ sink,
+                                    int kmaps) {
   const int t = blockIdx.x, hm = blockIdx.y;
   if (seq_len[tok_seq[t]] == 0) return;  // padding row
   const int rec = dv + 2;
   const float* p = partial + ((int64_t)t * HM + hm) * nsplit * rec;
   float w[MAXSPLIT];
-  float mx = -INFINITY;
+  const float sk = sink ? sink[hm / kmaps] : -INFINITY;
+  float mx = sk;
 #pragma unroll
   for (int z = 0; z < MAXSPLIT; z++) {
     w[z] = z < nsplit ? p[z * rec] : -INFINITY;
     mx = fmaxf(mx, w[z]);
   }
-  float lt = 0.f;
+  float lt = sink ? expf(sk - mx) : 0.f;
 #pragma unroll
   for (int z = 0; z < MAXSPLIT; z++) {
     w[z] = w[z] == -INFINITY ? 0.f : expf(w[z] - mx);
@@ -549,6 +567,30 @@ inline bool combo_ok(int KC, int DN, bool f32out) {
                     (KC == 18 && DN == 32));
 }
 
+void check_softmax_options(int64_t H, bool sigmoid, double softcap,
+                           const c10::optional<torch::Tensor>& dist_bias,
+                           const c10::optional<torch::Tensor>& sink) {
+  SEQ_CHECK(softcap >= 0.0 && !(sigmoid && (sink || softcap > 0.0)),
+            "soft cap / sink belong to the softmax form");
+  if (dist_bias)
+    SEQ_CHECK(dist_bias->scalar_type() == torch::kFloat &&
+                  dist_bias->is_contiguous() && dist_bias->dim() == 2 &&
+                  dist_bias->size(0) >= 1 && dist_bias->size(1) == H,
+              "distance bias fp32 [D + 1, H]");
+  if (sink)
+    SEQ_CHECK(sink->scalar_type() == torch::kFloat && sink->is_contiguous() &&
+                  sink->numel() == H, "sink fp32 [H]");
+}
+
+void set_softmax_options(MfmaArgs& a, double softcap,
+                         const c10::optional<torch::Tensor>& dist_bias,
+                         const c10::optional<torch::Tensor>& sink) {
+  a.softcap = (float)softcap;
+  a.dist_bias = dist_bias ? cptr<float>(*dist_bias) : nullptr;
+  a.dist_max = dist_bias ? (int)dist_bias->size(0) - 1 : 0;
+  a.sink = sink ? cptr<float>(*sink) : nullptr;
+}
+
 }  // namespace
 
 // Whether the matrix-core kernel covers these sizes (bf16 caches only).
@@ -574,9 +616,12 @@ void paged_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
                           double temp_coef, int64_t temp_every, int64_t kmaps,
                           int64_t window, int64_t keep_first,
                           c10::optional<torch::Tensor> head_bias,
-                          bool sigmoid) {
+                          bool sigmoid, double softcap,
+                          c10::optional<torch::Tensor> dist_bias,
+                          c10::optional<torch::Tensor> sink) {
   SEQ_CHECK(out.dim() == 4 && out.is_contiguous() && out.size(2) == kmaps,
             "mfma attention out [T, H, maps, dv]");
+  check_softmax_options(out.size(1), sigmoid, softcap, dist_bias, sink);
   SEQ_CHECK(keep_first >= 0, "kept first keys");
   if (head_bias)
     SEQ_CHECK(head_bias->scalar_type() == torch::kFloat &&
@@ -649,6 +694,7 @@ void paged_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
   a.keep_first = (int)keep_first;
   a.head_bias = head_bias ? cptr<float>(*head_bias) : nullptr;
   a.sigmoid = sigmoid ? 1 : 0;
+  set_softmax_options(a, softcap, dist_bias, sink);
   a.seq_len = nullptr; a.nsplit = 1; a.partial = nullptr;
   const int KC = pick_kc(dk), DN = pick_dn(dv);
   const dim3 grid(NT, H * kmaps);
@@ -668,13 +714,18 @@ void paged_attention_mfma_decode(torch::Tensor out, torch::Tensor partial,
                                  torch::Tensor page_table,
                                  torch::Tensor tok_seq, torch::Tensor positions,
                                  torch::Tensor seq_len, double scale,
+                                 double temp_coef, int64_t temp_every,
                                  int64_t kmaps, int64_t window,
                                  int64_t keep_first,
                                  c10::optional<torch::Tensor> head_bias,
-                                 bool sigmoid) {
+                                 bool sigmoid, double softcap,
+                                 c10::optional<torch::Tensor> dist_bias,
+                                 c10::optional<torch::Tensor> sink) {
   SEQ_CHECK(out.dim() == 4 && out.is_contiguous() && out.size(2) == kmaps &&
                 out.scalar_type() == torch::kFloat,
             "mfma decode out [T, H, maps, dv] fp32");
+  SEQ_CHECK(temp_every >= 1, "temperature period");
+  check_softmax_options(out.size(1), sigmoid, softcap, dist_bias, sink);
   SEQ_CHECK(keep_first >= 0, "kept first keys");
   if (head_bias)
     SEQ_CHECK(head_bias->scalar_type() == torch::kFloat &&
@@ -733,11 +784,14 @@ void paged_attention_mfma_decode(torch::Tensor out, torch::Tensor partial,
   a.tok_seq = cptr<int>(tok_seq); a.positions = cptr<int>(positions);
   a.r1 = nullptr; a.r2 = nullptr;
   a.H = H; a.G = G; a.dk = dk; a.dv = dv; a.ps = ps;
-  a.scale = (float)scale; a.temp_coef = 0.f; a.temp_every = 1; a.has_bias = 0;
+  a.scale = (float)scale; a.temp_coef = (float)temp_coef;
+  a.temp_every = (int)temp_every; a.has_bias = 0;
   a.kmaps = (int)kmaps; a.krow = krow; a.vrow = vrow; a.window = (int)window;
   a.keep_first = (int)keep_first;
   a.head_bias = head_bias ? cptr<float>(*head_bias) : nullptr;
   a.sigmoid = sigmoid ? 1 : 0;
+  set_softmax_options(a, softcap, dist_bias, sink);
+  a.sink = nullptr;  // the merge of the key splits adds the sink
   a.seq_len = cptr<int>(seq_len); a.nsplit = nsplit;
   a.partial = ptr<float>(partial);
   const int KC = pick_kc(dk), DN = pick_dn(dv);
@@ -750,7 +804,9 @@ void paged_attention_mfma_decode(torch::Tensor out, torch::Tensor partial,
                      dim3(dv <= 64 ? 64 : (dv <= 128 ? 128 : 256)), 0,
                      cur_stream(), ptr<float>(out), cptr<float>(partial),
                      cptr<int>(tok_seq), cptr<int>(seq_len), H * (int)kmaps,
-                     nsplit, dv, sigmoid ? 1 : 0);
+                     nsplit, dv, sigmoid ? 1 : 0,
+                     sink ? cptr<float>(*sink) : (const float*)nullptr,
+                     (int)kmaps);
 }
 
 void biased_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
@@ -765,5 +821,5 @@ void biased_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
   paged_attention_mfma(out.unsqueeze(2), proj, off_q, kcache, vcache,
                        page_table, tile_row0, tile_rows, max_tile_rows, tok_seq,
                        positions, r1, r2, scale, temp_coef, temp_every, 1, 0, 0,
-                       c10::nullopt, false);
+                       c10::nullopt, false, 0.0, c10::nullopt, c10::nullopt);
 }

@@ -54,7 +54,8 @@ void paged_attention_rows(Tensor out, Tensor proj, int64_t off_q, Tensor kcache,
                           OptTensor r2, double scale, double temp_coef,
                           int64_t temp_every, int64_t kmaps, int64_t window,
                           int64_t keep_first, OptTensor head_bias,
-                          bool sigmoid);
+                          bool sigmoid, double softcap, OptTensor dist_bias,
+                          OptTensor sink);
 void residual_layernorm(OptTensor out, Tensor res, OptTensor delta,
                         OptTensor post_w, double mult, OptTensor w, double eps);
 void xielu(Tensor out, Tensor x, Tensor pq);
@@ -80,7 +81,8 @@ void paged_attention_mfma(Tensor out, Tensor proj, int64_t off_q, Tensor kcache,
                           OptTensor r2, double scale, double temp_coef,
                           int64_t temp_every, int64_t kmaps, int64_t window,
                           int64_t keep_first, OptTensor head_bias,
-                          bool sigmoid);
+                          bool sigmoid, double softcap, OptTensor dist_bias,
+                          OptTensor sink);
 void biased_attention_mfma(Tensor out, Tensor proj, int64_t off_q,
                            Tensor kcache, Tensor vcache, Tensor page_table,
                            Tensor tile_row0, Tensor tile_rows,
@@ -92,9 +94,11 @@ void paged_attention_mfma_decode(Tensor out, Tensor partial, Tensor proj,
                                  int64_t off_q, Tensor kcache, OptTensor vcache,
                                  Tensor page_table, Tensor tok_seq,
                                  Tensor positions, Tensor seq_len, double scale,
+                                 double temp_coef, int64_t temp_every,
                                  int64_t kmaps, int64_t window,
                                  int64_t keep_first, OptTensor head_bias,
-                                 bool sigmoid);
+                                 bool sigmoid, double softcap,
+                                 OptTensor dist_bias, OptTensor sink);
 void residual_conv(Tensor out, Tensor x, Tensor w, Tensor conv_state,
                    Tensor tok_seq, Tensor seq_start, Tensor seq_len,
                    Tensor seq_slot, Tensor seq_pos0);
@@ -116,7 +120,31 @@ void moe_dispatch(Tensor rank, Tensor counts, Tensor idx);
 void moe_gather(Tensor xg, Tensor h, Tensor idx, Tensor rank, Tensor base,
                 int64_t E);
 void moe_combine(Tensor out, Tensor y, Tensor h, Tensor idx, Tensor wgt,
-                 Tensor rank, Tensor base, int64_t E, OptTensor shared);
+                 Tensor rank, Tensor base, int64_t E, OptTensor shared,
+                 OptTensor shared_gate);
+void embed_pair_hash(Tensor out, Tensor ids, Tensor embed, Tensor table,
+                     int64_t mul_prev, int64_t mul_cur, Tensor prev_state,
+                     Tensor tok_seq, Tensor seq_start, Tensor seq_len,
+                     Tensor seq_slot, Tensor seq_pos0);
+void stream_step(OptTensor out, Tensor xs, OptTensor delta, OptTensor mix,
+                 OptTensor out_w, double mult, OptTensor in_w, OptTensor norm_w,
+                 double eps);
+void rms_norm_cols(Tensor out, Tensor x, int64_t col, Tensor w, double eps);
+void rownorm_append(Tensor proj, int64_t nq, int64_t off_k, int64_t nk,
+                    int64_t off_v, int64_t nv, Tensor qw, OptTensor kw,
+                    double eps, OptTensor kcache, OptTensor vcache,
+                    Tensor slot_mapping);
+void heads_major(Tensor out, Tensor x);
+void heads_gate(Tensor out, Tensor o, Tensor gate);
+void ssd_scan(Tensor out, Tensor xbc, Tensor dt_raw, Tensor dt_bias,
+              Tensor A_log, Tensor D, Tensor state, Tensor seq_start,
+              Tensor seq_len, Tensor seq_slot, Tensor seq_pos0, int64_t G);
+void gated_group_norm(Tensor out, Tensor y, Tensor z, Tensor w, int64_t groups,
+                      double eps);
+void gelu_erf(Tensor out, Tensor x);
+void silu_glu(Tensor out, Tensor gate_up);
+void moe_route_topk(Tensor idx, Tensor wgt, Tensor logits, int64_t n,
+                    OptTensor bias);
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "dynamo_amd sequence-mixer kernels (gfx950)";
@@ -156,4 +184,15 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("moe_dispatch", &moe_dispatch);
   m.def("moe_gather", &moe_gather);
   m.def("moe_combine", &moe_combine);
+  m.def("embed_pair_hash", &embed_pair_hash);
+  m.def("stream_step", &stream_step);
+  m.def("rms_norm_cols", &rms_norm_cols);
+  m.def("rownorm_append", &rownorm_append);
+  m.def("heads_major", &heads_major);
+  m.def("heads_gate", &heads_gate);
+  m.def("ssd_scan", &ssd_scan);
+  m.def("gated_group_norm", &gated_group_norm);
+  m.def("gelu_erf", &gelu_erf);
+  m.def("silu_glu", &silu_glu);
+  m.def("moe_route_topk", &moe_route_topk);
 }

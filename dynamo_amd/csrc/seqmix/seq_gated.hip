@@ -389,7 +389,8 @@ __global__ void moe_combine_kernel(
     T* __restrict__ out, const T* __restrict__ y, const T* __restrict__ h,
     const int* __restrict__ idx, const float* __restrict__ wgt,
     const int* __restrict__ rank, const int* __restrict__ base,
-    const T* __restrict__ shared, int E, int W, int top, int rows) {
+    const T* __restrict__ shared, const float* __restrict__ shared_gate,
+    int gate_stride, int E, int W, int top, int rows) {
   constexpr int MAXTOP = 64;  // checked on the host
   __shared__ const T* src[MAXTOP];
   __shared__ float wj[MAXTOP];
@@ -407,10 +408,13 @@ __global__ void moe_combine_kernel(
     }
   }
   __syncthreads();
+  // the shared row weighs in with sigmoid(gate value of the token)
+  const float sg =
+      shared_gate ? sigmoid_f(shared_gate[(int64_t)t * gate_stride]) : 1.f;
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float acc = 0.f;
     for (int j = 0; j < top; j++) acc += wj[j] * to_f(src[j][c]);
-    if (shared) acc += to_f(shared[(int64_t)t * W + c]);
+    if (shared) acc += sg * to_f(shared[(int64_t)t * W + c]);
     out[(int64_t)t * W + c] = from_f<T>(acc);
   }
 }
@@ -622,8 +626,14 @@ void moe_gather(torch::Tensor xg, torch::Tensor h, torch::Tensor idx,
 void moe_combine(torch::Tensor out, torch::Tensor y, torch::Tensor h,
                  torch::Tensor idx, torch::Tensor wgt, torch::Tensor rank,
                  torch::Tensor base, int64_t E,
-                 c10::optional<torch::Tensor> shared) {
+                 c10::optional<torch::Tensor> shared,
+                 c10::optional<torch::Tensor> shared_gate) {
   const int T_ = h.size(0), W = h.size(1), top = idx.size(1);
+  if (shared_gate)
+    SEQ_CHECK(shared.has_value() && shared_gate->dim() == 1 &&
+                  shared_gate->size(0) == T_ &&
+                  shared_gate->scalar_type() == torch::kFloat,
+              "shared gate fp32 [T]");
   SEQ_CHECK(is_act(h) && h.dim() == 2 && h.is_contiguous() &&
                 out.is_contiguous() && out.dim() == 2 && out.size(0) == T_ &&
                 out.size(1) == W && out.scalar_type() == h.scalar_type() &&
@@ -646,6 +656,8 @@ void moe_combine(torch::Tensor out, torch::Tensor y, torch::Tensor h,
       moe_combine_kernel<T>, dim3(T_), dim3(pow2_block(W, 256)), 0,
       cur_stream(), ptr<T>(out), cptr<T>(y), cptr<T>(h), cptr<int>(idx),
       cptr<float>(wgt), cptr<int>(rank), cptr<int>(base),
-      shared ? cptr<T>(*shared) : (const T*)nullptr, (int)E, W, top,
+      shared ? cptr<T>(*shared) : (const T*)nullptr,
+      shared_gate ? cptr<float>(*shared_gate) : (const float*)nullptr,
+      shared_gate ? (int)shared_gate->stride(0) : 0, (int)E, W, top,
       (int)std::max<int64_t>(y.size(0), 1)););
 }

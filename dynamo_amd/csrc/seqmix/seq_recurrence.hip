@@ -467,6 +467,107 @@ __global__ void mlstm_nm_kernel(
        ? ((g).RT == 16 ? K<T, 1, 16> : K<T, 1, 32>)                          \
        : ((g).RT == 16 ? K<T, PEMAX, 16> : K<T, PEMAX, 32>))
 
+// ---------------------------------------------------------------------------
+// State-space recurrence with a scalar decay per head. Per token, with
+// dt = softplus(dt_raw + dt_bias) and a = exp(-exp(A_log) dt) from the
+// pre-pass: S <- a S + (dt B) x^T; o = S^T C + D x. B and C (state size dk)
+// are shared by the heads of a group; x is the head's dv value channels.
+template <typename T>
+__global__ void ssd_gates_kernel(float* __restrict__ out,  // [T, 2H]: dt | a
+                                 const T* __restrict__ dt_raw, int stride,
+                                 const float* __restrict__ dt_bias,
+                                 const float* __restrict__ A_log, int H,
+                                 int total) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int t = idx / H, hh = idx - t * H;
+  const float dt = softplus_f(to_f(dt_raw[(int64_t)t * stride + hh]) + dt_bias[hh]);
+  out[(int64_t)t * 2 * H + hh] = dt;
+  out[(int64_t)t * 2 * H + H + hh] = expf(-expf(A_log[hh]) * dt);
+}
+
+template <int PE, int RT>
+__global__ __launch_bounds__(512) void ssd_kernel(
+    float* __restrict__ out,          // [T, H, dv]
+    const float* __restrict__ xbc,    // [T, H*dv + 2*G*dk]: x | B | C
+    const float* __restrict__ gates,  // [T, 2H]: dt | decay
+    const float* __restrict__ Dskip,  // [H]
+    float* __restrict__ state,        // [slots, H, dk, dv]
+    SeqArgs sa, int H, int G, int dk, int dv, int KP) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  // [2 buffers][B | C][DKP]
+  const int DKP = KP * RT;
+  const int s = blockIdx.x, hh = blockIdx.y;
+  const int len = sa.seq_len[s];
+  if (len == 0) return;
+  const int start = sa.seq_start[s];
+  const bool fresh = sa.seq_pos0[s] == 0;
+  const int JW = 64 / KP;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int part = lane / JW;
+  const int nw = blockDim.x >> 6;
+  const int j = (blockIdx.z * nw + wave) * JW + (lane % JW);
+  const bool valid = j < dv;
+  float* sbase = state + ((int64_t)sa.seq_slot[s] * H + hh) * dk * dv;
+  float S[RT];
+  LOAD_STATE(S, sbase, fresh)
+  const int inner = H * dv, row = inner + 2 * G * dk;
+  const int grp = hh / (H / G);
+  const float dskip = Dskip[hh];
+  struct In { float b[PE], c[PE], xj, dt, a; };
+  In pre[DEPTH];
+  const int end = start + len;
+  auto fetch = [&](In& in, int t) {
+    const int64_t base = (int64_t)t * row + inner + grp * dk;
+#pragma unroll
+    for (int e = 0; e < PE; e++) {
+      const int i = threadIdx.x + e * blockDim.x;
+      in.b[e] = i < dk ? xbc[base + i] : 0.f;
+      in.c[e] = i < dk ? xbc[base + G * dk + i] : 0.f;
+    }
+    in.xj = valid ? xbc[(int64_t)t * row + hh * dv + j] : 0.f;
+    in.dt = gates[(int64_t)t * 2 * H + hh];
+    in.a = gates[(int64_t)t * 2 * H + H + hh];
+  };
+#pragma unroll
+  for (int u = 0; u < DEPTH; u++)
+    if (start + u < end) fetch(pre[u], start + u);
+  for (int t0 = start; t0 < end; t0 += DEPTH) {
+#pragma unroll
+    for (int u = 0; u < DEPTH; u++) {
+      const int t = t0 + u;
+      if (t >= end) break;
+      float* bl = lds + (u & 1) * 2 * DKP;
+      float* cl = bl + DKP;
+#pragma unroll
+      for (int e = 0; e < PE; e++) {
+        const int i = threadIdx.x + e * blockDim.x;
+        if (i < DKP) {
+          bl[i] = pre[u].b[e];
+          cl[i] = pre[u].c[e];
+        }
+      }
+      const float x_cur = pre[u].xj, a = pre[u].a;
+      const float dx = pre[u].dt * x_cur;
+      __syncthreads();
+      if (t + DEPTH < end) fetch(pre[u], t + DEPTH);
+      float br[RT], cr[RT];
+      READ_ROWS(br, bl)
+      READ_ROWS(cr, cl)
+      float o4[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int r = 0; r < RT; r++) {
+        S[r] = a * S[r] + br[r] * dx;
+        o4[r & 3] += cr[r] * S[r];
+      }
+      const float o = part_sum((o4[0] + o4[1]) + (o4[2] + o4[3]), JW);
+      if (valid && part == 0)
+        out[((int64_t)t * H + hh) * dv + j] = o + dskip * x_cur;
+    }
+  }
+  STORE_STATE(S, sbase)
+}
+
 #define PICK_KERNEL_F32(K, g)                                                \
   ((g).DKP <= (g).NW * 64                                                    \
        ? ((g).RT == 16 ? K<1, 16> : K<1, 32>)                                \
@@ -616,4 +717,43 @@ void mlstm_memory(torch::Tensor out, torch::Tensor proj, int64_t off_q,
         cptr<float>(gates), ptr<float>(state_n), ptr<float>(state_m), sa, H,
         dk);
   });
+}
+
+// xbc fp32 [T, H*dv + 2*G*dk] (x | B | C after convolution and activation),
+// dt_raw [T, >= H] in the activation type (any row stride), state
+// [slots, H, dk, dv]; out fp32 [T, H*dv].
+void ssd_scan(torch::Tensor out, torch::Tensor xbc, torch::Tensor dt_raw,
+              torch::Tensor dt_bias, torch::Tensor A_log, torch::Tensor D,
+              torch::Tensor state, torch::Tensor seq_start,
+              torch::Tensor seq_len, torch::Tensor seq_slot,
+              torch::Tensor seq_pos0, int64_t G) {
+  const int T_ = out.size(0);
+  SEQ_CHECK(state.dim() == 4 && state.scalar_type() == torch::kFloat &&
+                state.is_contiguous(), "ssd state [slots, H, N, P]");
+  const int H = state.size(1), dk = state.size(2), dv = state.size(3);
+  SEQ_CHECK(out.scalar_type() == torch::kFloat && out.is_contiguous() &&
+                out.dim() == 2 && out.size(1) == H * dv, "ssd out");
+  SEQ_CHECK(G >= 1 && H % G == 0, "ssd head grouping");
+  SEQ_CHECK(xbc.scalar_type() == torch::kFloat && xbc.is_contiguous() &&
+                xbc.size(0) == T_ && xbc.size(1) == H * dv + 2 * G * dk,
+            "ssd x | B | C");
+  SEQ_CHECK(is_act(dt_raw) && dt_raw.dim() == 2 && dt_raw.stride(1) == 1 &&
+                dt_raw.size(0) == T_ && dt_raw.size(1) >= H, "ssd dt");
+  for (const torch::Tensor* t : {&dt_bias, &A_log, &D})
+    SEQ_CHECK(t->scalar_type() == torch::kFloat && t->is_contiguous() &&
+                  t->numel() == H, "ssd head parameters");
+  const int B = seq_start.size(0);
+  if (T_ == 0 || B == 0) return;
+  SeqArgs sa = seq_args(seq_start, seq_len, seq_slot, seq_pos0, state.size(0));
+  Geometry g = geometry(dk, dv);
+  torch::Tensor gates = torch::empty({T_, 2 * H}, out.options());
+  DISPATCH_ACT(dt_raw, hipLaunchKernelGGL(
+      ssd_gates_kernel<T>, dim3((T_ * H + 255) / 256), dim3(256), 0,
+      cur_stream(), ptr<float>(gates), cptr<T>(dt_raw), (int)dt_raw.stride(0),
+      cptr<float>(dt_bias), cptr<float>(A_log), H, T_ * H););
+  hipLaunchKernelGGL(PICK_KERNEL_F32(ssd_kernel, g), dim3(B, H, g.tiles),
+                     dim3(g.NW * 64), 4 * g.DKP * sizeof(float), cur_stream(),
+                     ptr<float>(out), cptr<float>(xbc), cptr<float>(gates),
+                     cptr<float>(D), ptr<float>(state), sa, H, (int)G, dk, dv,
+                     g.KP);
 }

@@ -37,7 +37,7 @@ seq_sources = [
     os.path.join(SEQ, f)
     for f in ("seq_bindings.cpp", "seq_elementwise.hip", "seq_recurrence.hip",
               "seq_attention.hip", "seq_attention_mfma.hip", "seq_layer.hip",
-              "seq_gated.hip")
+              "seq_gated.hip", "seq_stream.hip")
 ]
 
 # hipcc emits packed-fp32 VALU ops from plain float code unless told not to
