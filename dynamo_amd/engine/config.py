@@ -169,6 +169,34 @@ PRESETS = {
     # layer-list model with an input convolution on every sublayer: sigmoid
     # attention under a window that keeps the first tokens, a minimal gated
     # recurrent unit, routed experts with identity and shared experts
+    "tiny-muzulorn": ModelConfig(
+        name="tiny-muzulorn", arch="muzulorn", hidden_size=64, vocab_size=150,
+        num_layers=4, rms_eps=1e-5, residual_mult=0.5, residual_streams=2,
+        pair_hash={"buckets": 97, "mul_prev": 31, "mul_cur": 5},
+        tie_embeddings=False, norm="rmsnorm", intermediate_size=0,
+        num_q_heads=1, num_kv_heads=1, head_dim=1,
+        layer_specs=[
+            {"type": "attention", "mixer": {
+                "heads": 4, "kv_heads": 2, "dim": 20, "vdim": 12,
+                "scale": 0.22, "softcap": 15.0, "bias_max": 48, "buckets": 12,
+                "q_temp": {"coef": 0.4, "every": 32}},
+             "mlp": {"kind": "moe", "expert": {"ff": 32},
+                     "router": {"experts": 4, "top": 2},
+                     "shared": {"ff": 48}}},
+            {"type": "latent_attention", "mixer": {
+                "heads": 3, "dim": 16, "rot_dim": 8, "vdim": 16,
+                "kv_rank": 24, "q_rank": 20, "scale": 0.2,
+                "mask": {"size": 24}, "rot": {"base": 10000.0, "dims": 8}},
+             "mlp": {"kind": "dense", "ff": 96}},
+            {"type": "mamba2", "mixer": {
+                "heads": 4, "vdim": 10, "state": 12, "groups": 2,
+                "norm_groups": 2, "conv": 3},
+             "mlp": None},
+            {"type": "attention", "mixer": {
+                "heads": 4, "kv_heads": 2, "dim": 20, "vdim": 12,
+                "scale": 0.22, "softcap": 15.0, "bias_max": 48, "buckets": 12,
+                "kv_from": 0},
+             "mlp": {"kind": "dense", "ff": 80}}]),
     "tiny-kefesun": ModelConfig(
         name="tiny-kefesun", arch="kefesun", hidden_size=80, vocab_size=150,
         num_layers=3, rms_eps=1e-5, embed_scale=3.0, conv_taps=3,

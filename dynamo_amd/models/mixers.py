@@ -883,6 +883,10 @@ class CappedAttention(torch.nn.Module):
         self.b_in = init.vec(self.off_v + self.nv, -0.2, 0.2).to(init.dtype)
         self.q_norm = init.vec(self.nq, 0.7, 1.3)
         self.k_norm = None if shared_cache else init.vec(self.nk, 0.7, 1.3)
+        # random weights: no more buckets than the largest distance allows
+        # (a checkpoint's table brings its own row count)
+        while buckets > 2 and not self.bias_max > buckets // 2:
+            buckets -= 1
         self.rel = init.vec((buckets, heads), -1.0, 1.0) if buckets else None
         self.w_o = init.mat(width, heads * vdim)
         self.b_o = init.vec(width, -0.2, 0.2).to(init.dtype)

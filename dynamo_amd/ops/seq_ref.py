@@ -621,7 +621,7 @@ def ssd_scan(xbc, dt_raw, dt_bias, A_log, D, state, sb, H, P, N, G):
     Bm = xbc[:, inner:inner + G * N].view(T, G, N)
     Cm = xbc[:, inner + G * N:inner + 2 * G * N].view(T, G, N)
     rep = H // G
-    dt = F.softplus(dt_raw.float() + dt_bias, threshold=20.0)      # [T, H]
+    dt = F.softplus(dt_raw[:, :H].float() + dt_bias, threshold=20.0)  # [T, H]
     decay = torch.exp(-torch.exp(A_log) * dt)
     out = torch.empty(T, H, P, dtype=torch.float32)
     for start, n, slot, pos0 in sb.spans():
