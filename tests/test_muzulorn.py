@@ -32,9 +32,16 @@ def full_ckpt(tmp_path_factory):
     return U.write_checkpoint(tmp_path_factory.mktemp("full"), cfg, W), cfg, W
 
 
+# in bf16 a router whose best two logits lie a rounding error apart may pick
+# the other expert; with one expert per token that moves a position by more
+# than any kernel fault would, so the bf16 comparison leaves that layout out
+CALM = [L if (L.get("mlp") or {}).get("router", {}).get("top") != 1
+        else U.with_mlp(L, U.DENSE) for L in FULL]
+
+
 @pytest.fixture(scope="module")
 def calm_ckpt(tmp_path_factory):
-    cfg = U.make_config(FULL)
+    cfg = U.make_config(CALM)
     W = U.random_weights(cfg, 1)
     U.calm_routers(W)
     return U.write_checkpoint(tmp_path_factory.mktemp("calm"), cfg, W), cfg, W
@@ -340,6 +347,11 @@ def test_mixed_batches_bf16(calm_ckpt):
     got = _run_plan(eng, toks, PLAN)
     for rid in ("a", "c", "e", "f"):
         assert U.close_bf16(got[rid], want[rid]), rid
+    # and each request alone, whole: the batch and the cut change nothing
+    # beyond the rounding of differently shaped matrix products
+    for rid in ("a", "c", "e"):
+        alone = U.replay(eng, rid + "-alone", toks[rid], [len(toks[rid])])
+        assert float(U.rel_err_rows(got[rid], alone).max()) < 0.03, rid
 
 
 # -- edges made visible ----------------------------------------------------------
