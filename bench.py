@@ -59,10 +59,10 @@ def parse_args():
                         "--mixer-model) beside Llama or Mixtral at equal "
                         "sizes (1 GPU)")
     p.add_argument("--mixer-model", default="bolatar",
-                   choices=["bolatar", "fironex", "kefesun"],
+                   choices=["bolatar", "fironex", "kefesun", "muzulorn"],
                    help="which layer-list design --mixer-compare measures")
     p.add_argument("--mixer-baseline", default=None,
-                   choices=["llama", "mixtral"],
+                   choices=["llama", "mixtral", "kefesun"],
                    help="the model beside it (default: mixtral for a design "
                         "with routed experts, else llama)")
     p.add_argument("--mixer-no-llama", action="store_true",

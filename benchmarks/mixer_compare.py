@@ -1,12 +1,12 @@
-"""Prefill and decode throughput of a layer-list design (Bolatar, Fironex
-or Kefesun) beside the dense-attention Llama layout - or, for a design with
+"""Prefill and decode throughput of a layer-list design (Bolatar, Fironex,
+Kefesun or Muzulorn) beside the dense-attention Llama layout - or, for a design with
 routed experts, the Mixtral layout - at equal width, depth, feed-forward
 size and vocabulary, random weights, one GPU, through the engine's own
 add_request/step loop (chunked prefill, then hipGraph decode).
 
     python bench.py --mixer-compare [--mixer-sizes small,medium]
-                    [--mixer-model bolatar|fironex|kefesun]
-                    [--mixer-baseline llama|mixtral]
+                    [--mixer-model bolatar|fironex|kefesun|muzulorn]
+                    [--mixer-baseline llama|mixtral|kefesun]
 
 Prints one JSON line: per size and model, prefill tokens/s (B prompts of
 ISL tokens until every request has its first token) and decode tokens/s
@@ -121,6 +121,51 @@ def kefesun_config(width, layers, ff):
                        num_kv_heads=1, head_dim=1)
 
 
+def muzulorn_config(width, layers, ff):
+    """Layer pattern: capped attention with a distance table (128-wide
+    heads, four query heads per kv head), latent attention under a
+    1024-token window (rank 512 + 64 rotated, queries through a latent of
+    three quarters of the width), a state-space layer (64-wide heads over
+    twice the width, state 128, eight groups), and a second attention layer
+    on the first one's keys and values; two residual streams; every layer
+    with eight gated experts of size ff / 2, two per token, and a gated
+    shared expert - the expert form and sizes of the Mixtral layout."""
+    from dynamo_amd.engine.config import ModelConfig
+    H = width // 128
+    mlp = {"kind": "moe", "expert": {"ff": ff // 2},
+           "router": {"experts": 8, "top": 2}, "shared": {"ff": ff // 2}}
+    attn = {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128,
+            "scale": 128 ** -0.5, "softcap": 30.0, "bias_max": 4096,
+            "buckets": 32, "q_temp": {"coef": 0.1, "every": 1024}}
+    lat = {"heads": H, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512,
+           "q_rank": 3 * width // 4, "scale": 192 ** -0.5,
+           "mask": {"size": 1024}, "rot": {"base": 10000.0, "dims": 64}}
+    sh = 2 * width // 64
+    ssm = {"heads": sh, "vdim": 64, "state": 128, "groups": min(8, sh),
+           "norm_groups": min(8, sh), "conv": 4}
+    specs = []
+    for i in range(layers):
+        k = i % 4
+        if k == 0:
+            specs.append({"type": "attention", "mlp": mlp, "mixer": attn})
+        elif k == 1:
+            specs.append({"type": "latent_attention", "mlp": mlp, "mixer": lat})
+        elif k == 2:
+            specs.append({"type": "mamba2", "mlp": mlp, "mixer": ssm})
+        else:
+            specs.append({"type": "attention", "mlp": mlp,
+                          "mixer": dict(attn, kv_from=i - 3)})
+    return ModelConfig(name=f"muzulorn-w{width}", arch="muzulorn",
+                       hidden_size=width, vocab_size=VOCAB, max_position=8192,
+                       num_layers=layers, rms_eps=1e-6, residual_mult=0.5,
+                       residual_streams=2,
+                       pair_hash={"buckets": 65521, "mul_prev": 31,
+                                  "mul_cur": 17},
+                       tie_embeddings=False, norm="rmsnorm",
+                       layer_specs=specs, intermediate_size=0, num_q_heads=1,
+                       num_kv_heads=1, head_dim=1)
+
+
 def mixtral_config(width, layers, ff):
     """Eight gated experts of size ff / 2, two per token: a token's active
     feed-forward weights equal a dense gated feed-forward of size ff."""
@@ -207,9 +252,11 @@ def run(sizes, device="cuda:0", model="bolatar", with_llama=True,
         baseline=None):
     res = {}
     make = {"bolatar": bolatar_config, "fironex": fironex_config,
-            "kefesun": kefesun_config}[model]
-    baseline = baseline or ("mixtral" if model == "kefesun" else "llama")
-    base = {"llama": llama_config, "mixtral": mixtral_config}[baseline]
+            "kefesun": kefesun_config, "muzulorn": muzulorn_config}[model]
+    baseline = baseline or ("mixtral" if model in ("kefesun", "muzulorn")
+                            else "llama")
+    base = {"llama": llama_config, "mixtral": mixtral_config,
+            "kefesun": kefesun_config}[baseline]
     for name in sizes:
         s = SIZES[name]
         args = (s["width"], s["layers"], s["ff"])

@@ -25,8 +25,8 @@
 // may be plain sigmoids of the scores (not normalised over the keys)
 // instead of a softmax. The softmax form further takes a soft cap
 // c tanh(score / c) on the scaled scores, a bias looked up by key distance
-// in a table [dist_max + 1, H] (added after the cap; distances beyond the
-// table take its last row), and a per-head sink: exp(sink_h) is added to the
+// in a table [H, dist_max + 1] (added after the cap; distances beyond the
+// table take its last entry), and a per-head sink: exp(sink_h) is added to the
 // softmax denominator, with no key and no value.
 #include "seq_common.h"
 
@@ -219,7 +219,8 @@ __global__ __launch_bounds__(1024) void biased_attention_kernel(
         x += __shfl_xor(x, 2, 64);
         if (softcap > 0.f) x = softcap * tanhf(x / softcap);
         if (has_bias) x -= b1[a] * log1pf(b2[a] * (float)(pos - jc));
-        if (dist_bias) x += dist_bias[min(pos - jc, dist_max) * H + h0 + a];
+        if (dist_bias)
+          x += dist_bias[(h0 + a) * (dist_max + 1) + min(pos - jc, dist_max)];
         x += hb[a];
         sc[p][a] = (j < ctx && (j >= jmin || j < keep_first)) ? x : -INFINITY;
       }
@@ -415,7 +416,7 @@ void launch_attention(torch::Tensor& out, torch::Tensor& proj, int64_t off_q,
       r1 ? 1 : 0, kmaps, vrow, window, keep_first,                          \
       head_bias ? cptr<float>(*head_bias) : nullptr, sigmoid ? 1 : 0,       \
       (float)softcap, dist_bias ? cptr<float>(*dist_bias) : nullptr,        \
-      dist_bias ? (int)dist_bias->size(0) - 1 : 0,                          \
+      dist_bias ? (int)dist_bias->size(1) - 1 : 0,                          \
       sink ? cptr<float>(*sink) : nullptr)
 #define LAUNCH_GS(GS_)                                                      \
   do {                                                                      \
@@ -484,8 +485,8 @@ void paged_attention_rows(torch::Tensor out, torch::Tensor proj, int64_t off_q,
   if (dist_bias)
     SEQ_CHECK(dist_bias->scalar_type() == torch::kFloat &&
                   dist_bias->is_contiguous() && dist_bias->dim() == 2 &&
-                  dist_bias->size(0) >= 1 && dist_bias->size(1) == out.size(1),
-              "distance bias fp32 [D + 1, H]");
+                  dist_bias->size(1) >= 1 && dist_bias->size(0) == out.size(1),
+              "distance bias fp32 [H, D + 1]");
   if (sink)
     SEQ_CHECK(sink->scalar_type() == torch::kFloat && sink->is_contiguous() &&
                   sink->numel() == out.size(1), "sink fp32 [H]");

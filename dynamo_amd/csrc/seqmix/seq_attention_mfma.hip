@@ -59,6 +59,12 @@ DEVINL float sigmoid_fast(float x) {
   return __builtin_amdgcn_rcpf(1.f + __expf(-x));
 }
 
+// tanh from the hardware exponential and reciprocal: 1 - 2 / (1 + e^(2x)),
+// exact at both ends (e^(2x) = 0 or inf)
+DEVINL float tanh_fast(float x) {
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __expf(2.f * x));
+}
+
 constexpr int BN = 64;    // keys per block
 constexpr int PADE = 8;   // padding elements per LDS row (16 bytes)
 
@@ -168,9 +174,11 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const float my_hb = !a.head_bias ? 0.f
                       : HEADS ? (my_ok ? a.head_bias[h + my_row] : 0.f)
                               : a.head_bias[h];
+  const float inv_cap = a.softcap > 0.f ? 1.f / a.softcap : 0.f;
   // head of this lane's row, for the tables indexed by head
   const int my_head = HEADS ? h + (my_ok ? my_row : 0) : h;
-  const float* my_dist = a.dist_bias ? a.dist_bias + my_head : nullptr;
+  const float* my_dist =
+      a.dist_bias ? a.dist_bias + (int64_t)my_head * (a.dist_max + 1) : nullptr;
   // prompt rows are in order; the heads of a token share its position
   const int kv_end = a.positions[HEADS ? row0 : row0 + nrows - 1] + 1;
   // the first key any row of the tile sees
@@ -355,10 +363,10 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
         for (int r = 0; r < 4; r++) {
           const int j = t0 + n * 16 + lg * 4 + r;
           float x = s[n][r] * my_qmul;
-          if (a.softcap > 0.f) x = a.softcap * tanhf(x / a.softcap);
+          if (a.softcap > 0.f) x = a.softcap * tanh_fast(x * inv_cap);
           x += my_hb;
           if (a.has_bias) x -= b1 * log1pf(b2 * (float)max(my_pos - j, 0));
-          if (my_dist) x += my_dist[min(max(my_pos - j, 0), a.dist_max) * H];
+          if (my_dist) x += my_dist[min(max(my_pos - j, 0), a.dist_max)];
           const bool seen = j <= my_pos && (window == 0 || j > my_pos - window ||
                                             j < a.keep_first);
           x = seen ? x : -INFINITY;
@@ -575,8 +583,8 @@ void check_softmax_options(int64_t H, bool sigmoid, double softcap,
   if (dist_bias)
     SEQ_CHECK(dist_bias->scalar_type() == torch::kFloat &&
                   dist_bias->is_contiguous() && dist_bias->dim() == 2 &&
-                  dist_bias->size(0) >= 1 && dist_bias->size(1) == H,
-              "distance bias fp32 [D + 1, H]");
+                  dist_bias->size(1) >= 1 && dist_bias->size(0) == H,
+              "distance bias fp32 [H, D + 1]");
   if (sink)
     SEQ_CHECK(sink->scalar_type() == torch::kFloat && sink->is_contiguous() &&
                   sink->numel() == H, "sink fp32 [H]");
@@ -587,7 +595,7 @@ void set_softmax_options(MfmaArgs& a, double softcap,
                          const c10::optional<torch::Tensor>& sink) {
   a.softcap = (float)softcap;
   a.dist_bias = dist_bias ? cptr<float>(*dist_bias) : nullptr;
-  a.dist_max = dist_bias ? (int)dist_bias->size(0) - 1 : 0;
+  a.dist_max = dist_bias ? (int)dist_bias->size(1) - 1 : 0;
   a.sink = sink ? cptr<float>(*sink) : nullptr;
 }
 

@@ -497,7 +497,11 @@ __global__ __launch_bounds__(512) void ssd_kernel(
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // [2 buffers][B | C][DKP]
   const int DKP = KP * RT;
-  const int s = blockIdx.x, hh = blockIdx.y;
+  // heads vary fastest over the workgroup index: workgroups go to the
+  // chip's eight dies in turn, and in a batch of decoded tokens beside a
+  // few prompt portions the long walks would otherwise all land on the
+  // dies that the portions' sequence numbers select
+  const int s = blockIdx.y, hh = blockIdx.x;
   const int len = sa.seq_len[s];
   if (len == 0) return;
   const int start = sa.seq_start[s];
@@ -751,7 +755,7 @@ void ssd_scan(torch::Tensor out, torch::Tensor xbc, torch::Tensor dt_raw,
       ssd_gates_kernel<T>, dim3((T_ * H + 255) / 256), dim3(256), 0,
       cur_stream(), ptr<float>(gates), cptr<T>(dt_raw), (int)dt_raw.stride(0),
       cptr<float>(dt_bias), cptr<float>(A_log), H, T_ * H););
-  hipLaunchKernelGGL(PICK_KERNEL_F32(ssd_kernel, g), dim3(B, H, g.tiles),
+  hipLaunchKernelGGL(PICK_KERNEL_F32(ssd_kernel, g), dim3(H, B, g.tiles),
                      dim3(g.NW * 64), 4 * g.DKP * sizeof(float), cur_stream(),
                      ptr<float>(out), cptr<float>(xbc), cptr<float>(gates),
                      cptr<float>(D), ptr<float>(state), sa, H, (int)G, dk, dv,

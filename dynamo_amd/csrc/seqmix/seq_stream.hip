@@ -245,27 +245,76 @@ __global__ void gated_group_norm_kernel(
 }
 
 // ---------------------------------------------------------------------------
-template <typename T>
+// 16-byte pieces of activations: 4 floats or 8 bf16
+template <typename T> struct Piece;
+template <> struct Piece<float> {
+  static constexpr int N = 4;
+  float4 v;
+  DEVINL float get(int i) const { return (&v.x)[i]; }
+  DEVINL void set(int i, float f) { (&v.x)[i] = f; }
+};
+template <> struct Piece<bf16_t> {
+  static constexpr int N = 8;
+  uint4 v;
+  DEVINL float get(int i) const {
+    const uint32_t w = (&v.x)[i >> 1];
+    union { float f; uint32_t u; } c;
+    c.u = (i & 1) ? (w & 0xffff0000u) : (w << 16);
+    return c.f;
+  }
+  DEVINL void set(int i, float f) {
+    uint32_t& w = (&v.x)[i >> 1];
+    const uint32_t b = from_f<bf16_t>(f);
+    w = (i & 1) ? ((w & 0x0000ffffu) | (b << 16)) : ((w & 0xffff0000u) | b);
+  }
+};
+
+DEVINL float gelu_erf_f(float v) {
+  return 0.5f * v * (1.f + erff(v * 0.70710678118654752440f));
+}
+
+// VEC: every thread one 16-byte piece (n counts pieces), else one element
+template <typename T, bool VEC>
 __global__ void gelu_erf_kernel(T* __restrict__ out, const T* __restrict__ x,
                                 int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const float v = to_f(x[i]);
-  out[i] = from_f<T>(0.5f * v * (1.f + erff(v * 0.70710678118654752440f)));
+  if (VEC) {
+    Piece<T> a, o;
+    a.v = reinterpret_cast<const decltype(a.v)*>(x)[i];
+#pragma unroll
+    for (int e = 0; e < Piece<T>::N; e++) o.set(e, gelu_erf_f(a.get(e)));
+    reinterpret_cast<decltype(o.v)*>(out)[i] = o.v;
+  } else {
+    out[i] = from_f<T>(gelu_erf_f(to_f(x[i])));
+  }
 }
 
 // gate_up [rows, 2F] -> out [rows, F] = silu(gate) * up
-template <typename T>
+template <typename T, bool VEC>
 __global__ void silu_glu_kernel(T* __restrict__ out,
                                 const T* __restrict__ gate_up, int F,
                                 int64_t n) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
-  const int64_t r = i / F;
-  const int c = i - r * F;
-  const float g = to_f(gate_up[r * 2 * F + c]);
-  const float u = to_f(gate_up[r * 2 * F + F + c]);
-  out[i] = from_f<T>(silu_f(g) * u);
+  if (VEC) {
+    constexpr int N = Piece<T>::N;
+    const int fp = F / N;  // pieces per output row
+    const int64_t r = i / fp;
+    const int c = (i - r * fp) * N;
+    Piece<T> g, u, o;
+    g.v = *reinterpret_cast<const decltype(g.v)*>(gate_up + r * 2 * F + c);
+    u.v = *reinterpret_cast<const decltype(u.v)*>(gate_up + r * 2 * F + F + c);
+#pragma unroll
+    for (int e = 0; e < N; e++) o.set(e, silu_f(g.get(e)) * u.get(e));
+    *reinterpret_cast<decltype(o.v)*>(out + r * F + c) = o.v;
+  } else {
+    const int64_t r = i / F;
+    const int c = i - r * F;
+    const float g = to_f(gate_up[r * 2 * F + c]);
+    const float u = to_f(gate_up[r * 2 * F + F + c]);
+    out[i] = from_f<T>(silu_f(g) * u);
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -549,9 +598,21 @@ void gelu_erf(torch::Tensor out, torch::Tensor x) {
                 out.numel() == x.numel(), "gelu rows");
   const int64_t n = x.numel();
   if (n == 0) return;
-  DISPATCH_ACT(x, hipLaunchKernelGGL(
-      gelu_erf_kernel<T>, dim3((n + 255) / 256), dim3(256), 0, cur_stream(),
-      ptr<T>(out), cptr<T>(x), n););
+  const bool al = reinterpret_cast<uintptr_t>(x.data_ptr()) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0;
+  DISPATCH_ACT(x, {
+    constexpr int N = Piece<T>::N;
+    if (al && n % N == 0) {
+      const int64_t np = n / N;
+      hipLaunchKernelGGL((gelu_erf_kernel<T, true>), dim3((np + 255) / 256),
+                         dim3(256), 0, cur_stream(), ptr<T>(out), cptr<T>(x),
+                         np);
+    } else {
+      hipLaunchKernelGGL((gelu_erf_kernel<T, false>), dim3((n + 255) / 256),
+                         dim3(256), 0, cur_stream(), ptr<T>(out), cptr<T>(x),
+                         n);
+    }
+  });
 }
 
 void silu_glu(torch::Tensor out, torch::Tensor gate_up) {
@@ -563,9 +624,21 @@ void silu_glu(torch::Tensor out, torch::Tensor gate_up) {
                 out.scalar_type() == gate_up.scalar_type(), "glu out");
   const int64_t n = out.numel();
   if (n == 0) return;
-  DISPATCH_ACT(gate_up, hipLaunchKernelGGL(
-      silu_glu_kernel<T>, dim3((n + 255) / 256), dim3(256), 0, cur_stream(),
-      ptr<T>(out), cptr<T>(gate_up), F, n););
+  const bool al = reinterpret_cast<uintptr_t>(gate_up.data_ptr()) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0;
+  DISPATCH_ACT(gate_up, {
+    constexpr int N = Piece<T>::N;
+    if (al && F % N == 0) {
+      const int64_t np = n / N;
+      hipLaunchKernelGGL((silu_glu_kernel<T, true>), dim3((np + 255) / 256),
+                         dim3(256), 0, cur_stream(), ptr<T>(out),
+                         cptr<T>(gate_up), F, np);
+    } else {
+      hipLaunchKernelGGL((silu_glu_kernel<T, false>), dim3((n + 255) / 256),
+                         dim3(256), 0, cur_stream(), ptr<T>(out),
+                         cptr<T>(gate_up), F, n);
+    }
+  });
 }
 
 void moe_route_topk(torch::Tensor idx, torch::Tensor wgt, torch::Tensor logits,

@@ -833,8 +833,9 @@ class RoutedExperts(torch.nn.Module):
 
 
 def distance_bias_table(rel: torch.Tensor, max_dist: int) -> torch.Tensor:
-    """fp32 [D + 1, H] from a bucketed table rel [B, H]: row n is the bias
-    of key distance n (the last row serves every distance >= D). Buckets:
+    """fp32 [H, D + 1] from a bucketed table rel [B, H]: column n is the
+    bias of key distance n (the last serves every distance >= D; a head's
+    distances lie side by side, as a tile of scores reads them). Buckets:
     n itself below B // 2; from there logarithmic steps that reach the last
     bucket at distance D = max_dist:
     min(B - 1, B//2 + floor(ln(n / (B//2)) / ln(D / (B//2)) * (B - B//2)))."""
@@ -849,7 +850,7 @@ def distance_bias_table(rel: torch.Tensor, max_dist: int) -> torch.Tensor:
             rows.append(min(B - 1, half + int(math.floor(
                 math.log(n / half) / math.log(max_dist / half) * (B - half)))))
     return rel.float()[torch.tensor(rows, dtype=torch.long,
-                                    device=rel.device)].contiguous()
+                                    device=rel.device)].t().contiguous()
 
 
 class CappedAttention(torch.nn.Module):

@@ -306,7 +306,7 @@ def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
     (not normalised over the keys). Further options of the softmax form: a
     query temperature 1 + temp_coef ln(floor((i + 1) / temp_every) + 1) on
     the scaled scores, a soft cap c tanh(score / c) after it, a bias by
-    distance dist_bias[min(i - j, D), h] (fp32 [D + 1, H]) added after the
+    distance dist_bias[h, min(i - j, D)] (fp32 [H, D + 1]) added after the
     cap, and a per-head sink (fp32 [H]): exp(sink_h) joins the softmax
     denominator without a key or value."""
     if q.is_cuda:

@@ -341,8 +341,8 @@ def paged_attention_rows(q, off_q, H, kmaps, kcache, vcache, dv, positions, sb,
             if softcap:
                 s = softcap * torch.tanh(s / softcap)
             if dist_bias is not None:
-                dist = (i - j).clamp(max=dist_bias.shape[0] - 1)
-                s = s + dist_bias[dist].t().view(H, 1, i + 1)
+                dist = (i - j).clamp(max=dist_bias.shape[1] - 1)
+                s = s + dist_bias[:, dist].view(H, 1, i + 1)
             if head_bias is not None:
                 s = s + head_bias.view(H, 1, 1)
             if sigmoid:
