@@ -83,13 +83,16 @@ struct MfmaArgs {
   float scale, temp_coef; int temp_every, has_bias;
   int kmaps, krow, vrow, window;
   int keep_first; const float* head_bias; int sigmoid;
-  float softcap; const float* dist_bias; int dist_max; const float* sink;
+  float softcap, inv_softcap; const float* dist_bias; int dist_max;
+  const float* sink;
   // HEADS mode: rows of a tile are heads of one decoded token
   const int* seq_len; int nsplit; float* partial;
 };
 
-// KC = padded key size / 32, DN = padded value size / 16
-template <int KC, int DN, typename TO, bool HEADS>
+// KC = padded key size / 32, DN = padded value size / 16. EX compiles the
+// soft cap and the distance table into the score loop; the variants for
+// wide latent rows have no registers to spare and are built without.
+template <int KC, int DN, typename TO, bool HEADS, bool EX>
 __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
     TO* __restrict__ out,  // [T, H, kmaps, dv]
     const MfmaArgs a) {
@@ -174,11 +177,9 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   const float my_hb = !a.head_bias ? 0.f
                       : HEADS ? (my_ok ? a.head_bias[h + my_row] : 0.f)
                               : a.head_bias[h];
-  const float inv_cap = a.softcap > 0.f ? 1.f / a.softcap : 0.f;
-  // head of this lane's row, for the tables indexed by head
-  const int my_head = HEADS ? h + (my_ok ? my_row : 0) : h;
-  const float* my_dist =
-      a.dist_bias ? a.dist_bias + (int64_t)my_head * (a.dist_max + 1) : nullptr;
+  // (the tables indexed by head are addressed where they are used, from
+  // kernel arguments: nothing of them stays in registers over the key loop
+  // when a layer has no such table - the widest variants have none to spare)
   // prompt rows are in order; the heads of a token share its position
   const int kv_end = a.positions[HEADS ? row0 : row0 + nrows - 1] + 1;
   // the first key any row of the tile sees
@@ -363,10 +364,14 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
         for (int r = 0; r < 4; r++) {
           const int j = t0 + n * 16 + lg * 4 + r;
           float x = s[n][r] * my_qmul;
-          if (a.softcap > 0.f) x = a.softcap * tanh_fast(x * inv_cap);
+          if (EX && a.softcap > 0.f)
+            x = a.softcap * tanh_fast(x * a.inv_softcap);
           x += my_hb;
           if (a.has_bias) x -= b1 * log1pf(b2 * (float)max(my_pos - j, 0));
-          if (my_dist) x += my_dist[min(max(my_pos - j, 0), a.dist_max)];
+          if (EX && a.dist_bias)
+            x += a.dist_bias[(HEADS ? h + (my_ok ? my_row : 0) : h) *
+                                 (a.dist_max + 1) +
+                             min(max(my_pos - j, 0), a.dist_max)];
           const bool seen = j <= my_pos && (window == 0 || j > my_pos - window ||
                                             j < a.keep_first);
           x = seen ? x : -INFINITY;
@@ -465,7 +470,7 @@ __global__ __launch_bounds__(256) void paged_attention_mfma_kernel(
   // ---- normalise and store query row lr, channels 16 d + 4 lg + r
   float inv = a.sigmoid ? 1.f : 1.f / l;
   if (a.sink) {  // exp(sink) joins the denominator
-    const float sk = a.sink[my_head];
+    const float sk = a.sink[h];  // prompt tiles: one head per workgroup
     const float mm = fmaxf(m, sk);
     const float c = expf(m - mm);
     inv = c / (l * c + expf(sk - mm));
@@ -526,16 +531,34 @@ inline size_t lds_bytes(int KC, int DN) {
          sizeof(short);
 }
 
-template <int KC, int DN, typename TO>
-void launch(dim3 grid, TO* out, const MfmaArgs& a) {
+inline bool score_extras(const MfmaArgs& a) {
+  return a.softcap > 0.f || a.dist_bias != nullptr;
+}
+
+template <int KC, int DN, typename TO, bool EX>
+void launch_ex(dim3 grid, TO* out, const MfmaArgs& a) {
   if (a.partial) {
     if constexpr (std::is_same<TO, float>::value)
-      hipLaunchKernelGGL((paged_attention_mfma_kernel<KC, DN, float, true>),
-                         grid, dim3(256), lds_bytes(KC, DN), cur_stream(), out,
-                         a);
+      hipLaunchKernelGGL(
+          (paged_attention_mfma_kernel<KC, DN, float, true, EX>), grid,
+          dim3(256), lds_bytes(KC, DN), cur_stream(), out, a);
   } else {
-    hipLaunchKernelGGL((paged_attention_mfma_kernel<KC, DN, TO, false>), grid,
-                       dim3(256), lds_bytes(KC, DN), cur_stream(), out, a);
+    hipLaunchKernelGGL((paged_attention_mfma_kernel<KC, DN, TO, false, EX>),
+                       grid, dim3(256), lds_bytes(KC, DN), cur_stream(), out,
+                       a);
+  }
+}
+
+template <int KC, int DN, typename TO>
+void launch(dim3 grid, TO* out, const MfmaArgs& a) {
+  if (score_extras(a)) {
+    if constexpr (KC <= 8 && KC != 6 && DN <= 16)
+      launch_ex<KC, DN, TO, true>(grid, out, a);
+    else
+      TORCH_CHECK(false, "seqmix: mfma attention sizes with a soft cap or "
+                         "distance table");
+  } else {
+    launch_ex<KC, DN, TO, false>(grid, out, a);
   }
 }
 
@@ -568,10 +591,10 @@ bool dispatch(int KC, int DN, dim3 grid, TO* out, const MfmaArgs& a) {
   return false;
 }
 
-inline bool combo_ok(int KC, int DN, bool f32out) {
+inline bool combo_ok(int KC, int DN, bool f32out, bool extras = false) {
   if (KC == 0 || DN == 0) return false;
   if (KC <= 8 && KC != 6 && DN <= 16) return true;
-  return f32out && ((KC == 6 && DN == 8) || (KC == 10 && DN == 16) ||
+  return !extras && f32out && ((KC == 6 && DN == 8) || (KC == 10 && DN == 16) ||
                     (KC == 18 && DN == 32));
 }
 
@@ -594,6 +617,7 @@ void set_softmax_options(MfmaArgs& a, double softcap,
                          const c10::optional<torch::Tensor>& dist_bias,
                          const c10::optional<torch::Tensor>& sink) {
   a.softcap = (float)softcap;
+  a.inv_softcap = softcap > 0.0 ? (float)(1.0 / softcap) : 0.f;
   a.dist_bias = dist_bias ? cptr<float>(*dist_bias) : nullptr;
   a.dist_max = dist_bias ? (int)dist_bias->size(1) - 1 : 0;
   a.sink = sink ? cptr<float>(*sink) : nullptr;
@@ -602,12 +626,14 @@ void set_softmax_options(MfmaArgs& a, double softcap,
 }  // namespace
 
 // Whether the matrix-core kernel covers these sizes (bf16 caches only).
-bool paged_attention_mfma_supported(int64_t dk, int64_t dv, bool f32out) {
+// `extras`: with a soft cap or a distance table (fewer sizes are built).
+bool paged_attention_mfma_supported(int64_t dk, int64_t dv, bool f32out,
+                                    bool extras) {
   if (dk % 8 || dv % 8 || dk < 8 || dv < 8) return false;
-  return combo_ok(pick_kc((int)dk), pick_dn((int)dv), f32out);
+  return combo_ok(pick_kc((int)dk), pick_dn((int)dv), f32out, extras);
 }
 bool biased_attention_mfma_supported(int64_t dk, int64_t dv) {
-  return paged_attention_mfma_supported(dk, dv, false);
+  return paged_attention_mfma_supported(dk, dv, false, false);
 }
 
 // Rows are given as tiles: tile i covers rows [tile_row0[i], + tile_rows[i])
@@ -661,7 +687,8 @@ void paged_attention_mfma(torch::Tensor out, torch::Tensor proj, int64_t off_q,
     vptr = cptr<bf16_t>(kcache);
     vrow = krow;
   }
-  SEQ_CHECK(paged_attention_mfma_supported(dk, dv, f32out),
+  SEQ_CHECK(paged_attention_mfma_supported(
+                dk, dv, f32out, softcap > 0.0 || dist_bias.has_value()),
             "mfma attention sizes");
   SEQ_CHECK(reinterpret_cast<uintptr_t>(kcache.data_ptr()) % 16 == 0 &&
                 reinterpret_cast<uintptr_t>(vptr) % 16 == 0 && krow % 8 == 0 &&
@@ -767,7 +794,9 @@ void paged_attention_mfma_decode(torch::Tensor out, torch::Tensor partial,
     vptr = cptr<bf16_t>(kcache);
     vrow = krow;
   }
-  SEQ_CHECK(paged_attention_mfma_supported(dk, dv, true), "mfma attention sizes");
+  SEQ_CHECK(paged_attention_mfma_supported(
+                dk, dv, true, softcap > 0.0 || dist_bias.has_value()),
+            "mfma attention sizes");
   SEQ_CHECK(reinterpret_cast<uintptr_t>(kcache.data_ptr()) % 16 == 0 &&
                 reinterpret_cast<uintptr_t>(vptr) % 16 == 0 && krow % 8 == 0 &&
                 vrow % 8 == 0, "mfma attention cache alignment");

@@ -73,7 +73,8 @@ void rglru_scan(Tensor out, Tensor u, Tensor gates, Tensor br, Tensor bi,
                 Tensor seq_len, Tensor seq_slot, Tensor seq_pos0, double decay,
                 int64_t max_len);
 bool biased_attention_mfma_supported(int64_t dk, int64_t dv);
-bool paged_attention_mfma_supported(int64_t dk, int64_t dv, bool f32out);
+bool paged_attention_mfma_supported(int64_t dk, int64_t dv, bool f32out,
+                                    bool extras);
 void paged_attention_mfma(Tensor out, Tensor proj, int64_t off_q, Tensor kcache,
                           OptTensor vcache, Tensor page_table, Tensor tile_row0,
                           Tensor tile_rows, int64_t max_tile_rows,

@@ -319,8 +319,10 @@ def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
         # other sizes and the remaining rows take the row kernel.
         krow, G = kcache.shape[3], kcache.shape[1]
         f32out = out_dtype == torch.float32
+        extras = softcap > 0 or dist_bias is not None
         fits = (q.dtype == torch.bfloat16
-                and m.paged_attention_mfma_supported(krow // kmaps, dv, f32out)
+                and m.paged_attention_mfma_supported(krow // kmaps, dv, f32out,
+                                                     extras)
                 and krow % 8 == 0 and kcache.data_ptr() % 16 == 0
                 and (vcache is None or vcache.data_ptr() % 16 == 0))
         tiled = fits and sb.tiles is not None
@@ -330,7 +332,8 @@ def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
                 float(softcap), dist_bias, sink)
         temp = (float(temp_coef), int(temp_every))
         if (fits and ndec and H // G >= 8 and f32out
-                and m.paged_attention_mfma_supported(krow // kmaps, dv, True)):
+                and m.paged_attention_mfma_supported(krow // kmaps, dv, True,
+                                                     extras)):
             nsplit = max(1, min(16, 512 // (ndec * G * kmaps)))
             part = torch.empty(ndec, H, kmaps, nsplit, dv + 2,
                                dtype=torch.float32, device=q.device)
