@@ -538,6 +538,61 @@ def test_large_heads_bf16_on_the_matrix_cores(tmp_path):
         assert U.close_bf16(got, want), sizes
 
 
+OTHER = [   # another order: state-space first, shared layers of both kinds
+    {"type": "mamba2",
+     "mixer": {"heads": 5, "vdim": 32, "state": 24, "groups": 1,
+               "norm_groups": 5, "conv": 2},
+     "mlp": {"kind": "dense", "ff": 200}},
+    {"type": "latent_attention",
+     "mixer": {"heads": 8, "dim": 48, "rot_dim": 16, "vdim": 40,
+               "kv_rank": 96, "q_rank": 64, "scale": 0.13,
+               "mask": {"size": 65}, "rot": {"base": 50000.0, "dims": 16}},
+     "mlp": {"kind": "moe", "expert": {"ff": 48},
+             "router": {"experts": 6, "top": 3}, "shared": {"ff": 24}}},
+    {"type": "attention",
+     "mixer": {"heads": 5, "kv_heads": 5, "dim": 32, "vdim": 48,
+               "scale": 0.18, "softcap": 12.0, "bias_max": 100,
+               "q_temp": {"coef": 1.1, "every": 64}},
+     "mlp": None},
+    {"type": "latent_attention",
+     "mixer": {"heads": 8, "dim": 48, "rot_dim": 16, "vdim": 40,
+               "kv_rank": 96, "q_rank": 64, "scale": 0.13, "kv_from": 1,
+               "mask": {"size": 130}, "rot": {"base": 50000.0, "dims": 16}},
+     "mlp": {"kind": "dense", "ff": 120}},
+    {"type": "attention",
+     "mixer": {"heads": 5, "kv_heads": 5, "dim": 32, "vdim": 48,
+               "scale": 0.18, "bias_max": 100, "kv_from": 2},
+     "mlp": {"kind": "moe", "expert": {"ff": 48},
+             "router": {"experts": 6, "top": 3}, "shared": {"ff": 24}}}]
+
+
+@pytest.mark.parametrize("device", DEVICES)
+def test_other_layout_on_64_token_pages(tmp_path, device):
+    """Another layer order and other sizes on the page size the replay
+    command uses: windows of one page + 1 and two pages + 2 (the shared
+    latent layer has a window of its own on the other layer's rows), a
+    shared attention layer without cap and temperature on capped keys, 24
+    bias buckets, three streams; a 200-token prompt whole, cut at and
+    around page borders, and decoded; in bf16 on the GPU as well."""
+    def edit(W):
+        for k in W:
+            if k.endswith(".router"):
+                W[k] = (W[k].float() * 6).to(W[k].dtype)
+    path, cfg, W = _case(tmp_path, OTHER, seed=21, rel_rows=24, width=160,
+                         vocab=211, streams=3, mult=0.7,
+                         bigram=(257, 1009, 13), edit=edit)
+    toks = U.tokens_for(cfg, 200, 21)
+    eng = U.make_engine(path, device, pages=8, page_size=64, slots=2)
+    plans = [[200], [63, 2, 63, 1], [64, 64, 3, 1]]
+    want = _check(eng, cfg, W, toks, plans)
+    if device != "cpu":
+        eng = U.make_engine(path, device, dtype="bfloat16", pages=8,
+                            page_size=64, slots=2)
+        for k, sizes in enumerate(plans):
+            got = U.replay(eng, f"b{k}", toks, sizes)
+            assert U.close_bf16(got, want), sizes
+
+
 def test_bad_configs_are_refused(tmp_path):
     from dynamo_amd.models.registry import build_model, resolve_model_config
     bad = copy.deepcopy(U.ATTN)
