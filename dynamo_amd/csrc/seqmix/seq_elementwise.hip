@@ -68,7 +68,10 @@ __global__ void causal_conv_kernel(
   const int start = seq_start[s], pos0 = seq_pos0[s];
   const float* st = conv_state + (int64_t)seq_slot[s] * (taps - 1) * C;
   const int rel = t - start;  // rows of this portion before t
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+  // one thread per (token, channel): the loads of a row's channels issue
+  // together instead of in a workgroup's loop over the row
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c < C) {
     float acc = bias ? bias[c] : 0.f;
     for (int j = 0; j < taps; j++) {
       const int back = taps - 1 - j;  // how many tokens before t
@@ -432,8 +435,8 @@ void causal_conv(torch::Tensor out, torch::Tensor x, torch::Tensor w,
   check_seq(seq_pos0, B, "seq_pos0");
   if (T_ == 0) return;
   DISPATCH_ACT(x, {
-    hipLaunchKernelGGL(causal_conv_kernel<T>, dim3(T_), dim3(row_block(C)),
-                       0, cur_stream(), ptr<float>(out), cptr<T>(x),
+    hipLaunchKernelGGL(causal_conv_kernel<T>, dim3(T_, (C + 255) / 256),
+                       dim3(256), 0, cur_stream(), ptr<float>(out), cptr<T>(x),
                        (int)x.stride(0), cptr<float>(w),
                        bias ? cptr<float>(*bias) : (const float*)nullptr,
                        silu ? 1 : 0, cptr<float>(conv_state),

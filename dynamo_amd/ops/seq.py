@@ -334,7 +334,9 @@ def paged_attention_rows(q, off_q: int, H: int, kmaps: int, kcache, vcache,
         if (fits and ndec and H // G >= 8 and f32out
                 and m.paged_attention_mfma_supported(krow // kmaps, dv, True,
                                                      extras)):
-            nsplit = max(1, min(16, 512 // (ndec * G * kmaps)))
+            # about one workgroup per compute unit: more key splits only
+            # add staging and merge work (measured with and without a window)
+            nsplit = max(1, min(16, 256 // (ndec * G * kmaps)))
             part = torch.empty(ndec, H, kmaps, nsplit, dv + 2,
                                dtype=torch.float32, device=q.device)
             m.paged_attention_mfma_decode(
