@@ -60,7 +60,8 @@ def build_mixer(kind: str, m: dict, width: int, eps: float, init: _Init):
             width, m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["scale"],
             eps, init, temp_coef=temp.get("coef", 0.0),
             temp_every=temp.get("every", 1), softcap=m.get("softcap", 0.0),
-            buckets=m.get("buckets", 16) if "bias_max" in m else 0,  # the checkpoint table's rows win
+            # a checkpoint's table brings its own row count
+            buckets=m.get("buckets", 32) if "bias_max" in m else 0,
             bias_max=m.get("bias_max", 0), shared_cache=shared)
     if kind == "latent_attention":
         return LatentAttention(
